@@ -1,0 +1,167 @@
+/*
+ * mops_hip.h — C ABI of libmops_hip.so: hand-written gfx950 (MI355X) kernels for the hot operators of
+ * the `mops` operator library of nano_vllm_ninetoothed.
+ *
+ * Conventions for every launcher below
+ *   - all pointers are DEVICE pointers unless stated; activations/caches/weights are bf16 (raw 16-bit
+ *     words), metadata is int32 unless a flag says otherwise;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); the launch is asynchronous,
+ *     nothing synchronises, nothing is allocated, nothing is freed;
+ *   - return value: MOPS_HIP_OK (0) or a negative MOPS_HIP_E* status; on a negative status no kernel was
+ *     launched.  Argument validation (null pointers, unsupported sizes, misalignment) happens on the host
+ *     before launch, mirroring the reference's wrapper-side `assert`s.
+ *
+ * The reference has no native code: each entry point replaces the GPU kernel(s) behind one op name of
+ * the reference's registry (mops/__init__.py:15-26), cited per function.
+ */
+#ifndef MOPS_HIP_H
+#define MOPS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOPS_HIP_OK 0
+#define MOPS_HIP_EINVAL (-1)       /* null pointer, negative size, inconsistent arguments            */
+#define MOPS_HIP_EUNSUPPORTED (-2) /* shape the kernels are not written for (head_dim, block size…)  */
+#define MOPS_HIP_EALIGN (-3)       /* pointer or stride breaks the 16-byte alignment the kernels need */
+#define MOPS_HIP_EWORKSPACE (-4)   /* workspace missing or smaller than mops_hip_*_workspace_bytes    */
+#define MOPS_HIP_ELAUNCH (-5)      /* hipLaunchKernel reported an error (see mops_hip_last_hip_error) */
+
+/* ABI version of this header; bumped on any signature change. */
+int mops_hip_abi_version(void);
+
+/* Static, human-readable text for a status returned by any function here. */
+const char* mops_hip_status_string(int status);
+
+/* hipError_t (as int) of the last failed launch on this host thread, 0 if none. */
+int mops_hip_last_hip_error(void);
+
+/*
+ * store_kvcache — slot_mapping scatter of freshly computed K and V rows into the paged cache.
+ * Replaces: mops/triton/attention.py:7-38 (store_kvcache_kernel + wrapper), reached from
+ * mops/torch/ops.py:62-65 and called at nanovllm/layers/attention.py:29.
+ *
+ *   for i in [0, n_tokens): s = slot_mapping[i]; if s == -1 skip;
+ *       k_cache[s*row_elems : (s+1)*row_elems] = key[i*key_row_stride : +row_elems]   (same for V)
+ *
+ * key/value: rows of row_elems (= num_kv_heads*head_dim) contiguous bf16, row i at element offset
+ * i*{key,value}_row_stride (strides in ELEMENTS, may exceed row_elems: V is a view into the qkv buffer).
+ * k_cache/v_cache: contiguous [num_slots, row_elems].  Slots outside [0, num_slots) other than -1 are
+ * skipped as well (the reference would write out of bounds).  Bit-exact copy.
+ * Needs row_elems % 8 == 0, strides % 8 == 0 and 16-byte aligned base pointers.
+ */
+int mops_hip_store_kvcache(const void* key, int64_t key_row_stride,
+                           const void* value, int64_t value_row_stride,
+                           void* k_cache, void* v_cache,
+                           const int32_t* slot_mapping,
+                           int64_t n_tokens, int64_t row_elems, int64_t num_slots,
+                           void* stream);
+
+/*
+ * embedding — row gather out[i, :] = weight[ids[i], :].
+ * Replaces: mops/torch/ops.py:57-59 (F.embedding), mops/triton/embedding.py:6-50; called at
+ * nanovllm/layers/embed_head.py:41.
+ * ids: n_ids indices, int64 when ids_are_int64 != 0 else int32.  weight: [vocab, hidden] bf16 with row
+ * stride weight_row_stride (elements).  out: contiguous [n_ids, hidden].  An id outside [0, vocab)
+ * produces a zero row instead of a fault.  Bit-exact copy.  hidden % 8 == 0, stride % 8 == 0.
+ */
+int mops_hip_embedding(const void* ids, int ids_are_int64,
+                       const void* weight, int64_t weight_row_stride,
+                       void* out,
+                       int64_t n_ids, int64_t vocab, int64_t hidden,
+                       void* stream);
+
+/*
+ * rms_forward — y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w), fp32 statistics, two bf16 roundings.
+ * Replaces: mops/torch/ops.py:9-16, mops/triton/rms_forward.py:7-36; called at
+ * nanovllm/layers/layernorm.py:21 (2-D hidden states and the 3-D strided q/k views of
+ * nanovllm/models/qwen3.py:76-77).
+ * x is addressed as x[(o*stride_outer + i*stride_inner) + 0..n) for o < rows_outer, i < rows_inner
+ * (strides in elements); y is contiguous [rows_outer*rows_inner, n]; x is never written.
+ * n % 8 == 0, n <= 16384, strides % 8 == 0.
+ */
+int mops_hip_rms_forward(const void* x, const void* weight, void* y,
+                         int64_t rows_outer, int64_t rows_inner, int64_t n,
+                         int64_t stride_outer, int64_t stride_inner,
+                         float eps, void* stream);
+
+/*
+ * add_rms_forward — s = float(x) + float(residual); residual_out = bf16(s);
+ *                   y = bf16(bf16(s * rsqrt(mean(s^2) + eps)) * w)   (statistics on the unrounded s).
+ * Replaces: mops/torch/ops.py:18-30, mops/triton/add_rms_forward.py:7-39; called at
+ * nanovllm/layers/layernorm.py:29.
+ * x, residual: [rows, n] with row strides x_row_stride / residual_row_stride (elements); y and
+ * residual_out contiguous [rows, n].  residual_out may alias residual (in-place convention of the
+ * triton/ninetoothed backends) when residual is contiguous; y must not alias an input.
+ */
+int mops_hip_add_rms_forward(const void* x, int64_t x_row_stride,
+                             const void* residual, int64_t residual_row_stride,
+                             const void* weight,
+                             void* y, void* residual_out,
+                             int64_t rows, int64_t n,
+                             float eps, void* stream);
+
+/*
+ * Paged decode attention (one query token per sequence against the block-table-addressed KV cache).
+ * Replaces: flash_attn.flash_attn_with_kvcache as reached from mops/torch/ops.py:74-76 (semantics
+ * spelled out in the commented torch version at mops/torch/ops.py:78-125) and the NineToothed kernel
+ * mops/ninetoothed/attention.py:157-348; called at nanovllm/layers/attention.py:40-42.
+ *
+ *   out[b,h,:] = softmax_t( scale * q[b,h,:] . K[b,t,h/(hq/hkv),:] ) @ V[b,t,h/(hq/hkv),:],
+ *   t in [0, cache_seqlens[b]),  token t at cache[block_table[b, t/block_size], t%block_size, kvhead, :]
+ *
+ * q: [batch, hq, 128] bf16, batch stride q_batch_stride elements (head stride 128).
+ * k_cache/v_cache: contiguous [num_blocks, block_size, hkv, 128] bf16.
+ * block_table: int32 [batch, *] with row stride block_table_row_stride, at least
+ * max_blocks_per_seq columns; columns at or beyond ceil(cache_seqlens[b]/block_size) are never read
+ * (they hold -1); an entry outside [0, num_blocks) inside the used range is treated as an empty block.
+ * cache_seqlens[b] is clamped to [0, max_blocks_per_seq*block_size]; 0 gives a zero output row.
+ * out: contiguous [batch, hq, 128] bf16.
+ * workspace: device scratch of at least mops_hip_paged_decode_workspace_bytes(...) bytes, 256-byte
+ * aligned, private to this call until it completes on `stream`.
+ * Supported: head_dim 128, block_size a multiple of 32, hq/hkv in {1,2,4,8,16}.
+ */
+int64_t mops_hip_paged_decode_workspace_bytes(int64_t batch, int64_t hq, int64_t hkv,
+                                              int64_t max_blocks_per_seq, int64_t block_size);
+
+int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
+                                    const void* k_cache, const void* v_cache,
+                                    const int32_t* cache_seqlens,
+                                    const int32_t* block_table, int64_t block_table_row_stride,
+                                    void* out,
+                                    int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                    int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                    float softmax_scale,
+                                    void* workspace, int64_t workspace_bytes,
+                                    void* stream);
+
+/*
+ * Varlen (packed, THD) causal prefill attention with grouped-query heads.
+ * Replaces: flash_attn.flash_attn_varlen_func as reached from mops/torch/ops.py:70-72 and the Triton
+ * kernel mops/triton/attention.py:42-146; called at nanovllm/layers/attention.py:34-37.
+ *
+ *   for sequence s with tokens [cu_seqlens[s], cu_seqlens[s+1]):
+ *     out[i,h,:] = softmax_{j<=i}( scale * q[i,h,:] . k[j,h/(hq/hkv),:] ) @ v[j,h/(hq/hkv),:]
+ *
+ * q/k/v/out: [total_tokens, heads, 128] bf16 with per-tensor token strides (elements) and head stride
+ * 128; cu_seqlens: int32 [batch+1], cu_seqlens[0] == 0, non-decreasing, last == total_tokens
+ * (q and k share it: no prefix-cache path here).  max_seqlen bounds every sequence length and only
+ * sizes the launch.  Sequences of length 0 are allowed.
+ */
+int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_stride,
+                                     const void* k, int64_t k_token_stride,
+                                     const void* v, int64_t v_token_stride,
+                                     void* out, int64_t out_token_stride,
+                                     const int32_t* cu_seqlens,
+                                     int64_t batch, int64_t total_tokens, int64_t max_seqlen,
+                                     int64_t hq, int64_t hkv, int64_t head_dim,
+                                     float softmax_scale,
+                                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOPS_HIP_H */

@@ -1,0 +1,262 @@
+"""The `hip` backend: the six hot operators run hand-written gfx950 kernels through the C ABI of
+libmops_hip.so; the remaining names are library-torch delegates so that the engine's layers resolve.
+
+Every function keeps the name and call form the reference's layers use (nanovllm/layers/attention.py:29-42,
+layernorm.py:21,29, embed_head.py:41).  Wrappers validate layouts with exceptions before launching
+(the reference asserts in its wrappers, mops/triton/attention.py:34-37), allocate outputs with the torch
+allocator, launch on the current torch stream and never synchronise.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ... import _capi
+from .registry import register_hip_op
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _require_cuda_bf16(name: str, t: torch.Tensor) -> None:
+    _require(t.is_cuda, f"{name} must live on the GPU")
+    _require(t.dtype == torch.bfloat16, f"{name} must be bfloat16, got {t.dtype}")
+
+
+# ----------------------------------------------------------------------------------------------------
+# hot ops: HIP kernels
+# ----------------------------------------------------------------------------------------------------
+
+@register_hip_op
+def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slot_mapping: torch.Tensor) -> None:
+    """Scatter of K/V rows into the paged cache; layout rules of mops/triton/attention.py:30-38."""
+    _require(key.dim() == 3 and value.shape == key.shape, "key/value must be [N, num_kv_heads, head_dim]")
+    n, num_heads, head_dim = key.shape
+    d = num_heads * head_dim
+    for name, t in (("key", key), ("value", value), ("k_cache", k_cache), ("v_cache", v_cache)):
+        _require_cuda_bf16(name, t)
+    _require(key.stride(-1) == 1 and value.stride(-1) == 1, "key/value last dim must be contiguous")
+    _require(key.stride(1) == head_dim and value.stride(1) == head_dim, "key/value head stride must be head_dim")
+    _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape, "caches must be [blocks, block_size, heads, dim]")
+    _require(k_cache.stride(1) == d and v_cache.stride(1) == d, "cache token stride must be num_kv_heads*head_dim")
+    _require(k_cache.is_contiguous() and v_cache.is_contiguous(), "caches must be contiguous")
+    _require(slot_mapping.numel() == n, "slot_mapping must have one entry per token")
+    _require(slot_mapping.dtype == torch.int32 and slot_mapping.is_cuda and slot_mapping.is_contiguous(),
+             "slot_mapping must be a contiguous int32 GPU tensor")
+    lib = _capi.load()
+    num_slots = k_cache.shape[0] * k_cache.shape[1]
+    st = lib.mops_hip_store_kvcache(key.data_ptr(), key.stride(0) if n > 1 else max(key.stride(0), d),
+                                    value.data_ptr(), value.stride(0) if n > 1 else max(value.stride(0), d),
+                                    k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
+                                    n, d, num_slots, _stream(key))
+    _capi.check("mops_hip_store_kvcache", st)
+
+
+@register_hip_op
+def embedding(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """Row gather with the result shape of F.embedding (mops/torch/ops.py:57-59)."""
+    _require_cuda_bf16("weight", weight)
+    _require(weight.dim() == 2 and weight.stride(1) == 1, "weight must be [vocab, hidden] with contiguous rows")
+    _require(x.is_cuda and x.dtype in (torch.int32, torch.int64), "ids must be an int32/int64 GPU tensor")
+    ids = x if x.is_contiguous() else x.contiguous()
+    vocab, hidden = weight.shape
+    out = torch.empty((*x.shape, hidden), dtype=weight.dtype, device=weight.device)
+    lib = _capi.load()
+    st = lib.mops_hip_embedding(ids.data_ptr(), 1 if ids.dtype == torch.int64 else 0, weight.data_ptr(),
+                                weight.stride(0), out.data_ptr(), ids.numel(), vocab, hidden, _stream(weight))
+    _capi.check("mops_hip_embedding", st)
+    return out
+
+
+def _row_view(x: torch.Tensor):
+    """Describes x[..., n] as rows_outer x rows_inner rows with two element strides, or returns None."""
+    n = x.shape[-1]
+    if x.stride(-1) != 1 and n > 1:
+        return None
+    lead = [(s, st) for s, st in zip(x.shape[:-1], x.stride()[:-1]) if s != 1]
+    # merge adjacent leading dims that are contiguous with each other
+    merged: list[list[int]] = []
+    for size, stride in lead:
+        if merged and merged[-1][1] == stride * size:
+            merged[-1][0] *= size
+            merged[-1][1] = stride
+        else:
+            merged.append([size, stride])
+    if len(merged) == 0:
+        return 1, 1, n, n
+    if len(merged) == 1:
+        return 1, merged[0][0], 0, merged[0][1]
+    if len(merged) == 2:
+        return merged[0][0], merged[1][0], merged[0][1], merged[1][1]
+    return None
+
+
+@register_hip_op
+def rms_forward(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMSNorm returning a new tensor (mops/torch/ops.py:9-16); strided 3-D views are read in place."""
+    _require_cuda_bf16("x", x)
+    _require_cuda_bf16("weight", weight)
+    n = x.shape[-1]
+    _require(weight.dim() == 1 and weight.shape[0] == n and weight.is_contiguous(), "weight must be [n] contiguous")
+    view = _row_view(x) if x.numel() else (0, 0, 0, 0)
+    if view is None:
+        x = x.contiguous()
+        view = _row_view(x)
+    rows_outer, rows_inner, stride_outer, stride_inner = view
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    lib = _capi.load()
+    st = lib.mops_hip_rms_forward(x.data_ptr(), weight.data_ptr(), y.data_ptr(), rows_outer, rows_inner, n,
+                                  stride_outer, stride_inner, float(eps), _stream(x))
+    _capi.check("mops_hip_rms_forward", st)
+    return y
+
+
+@register_hip_op
+def add_rms_forward(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float):
+    """Fused residual add + RMSNorm; returns (y, new_residual) as new tensors (mops/torch/ops.py:18-30)."""
+    _require_cuda_bf16("x", x)
+    _require_cuda_bf16("residual", residual)
+    _require_cuda_bf16("weight", weight)
+    _require(x.shape == residual.shape, "x and residual must have the same shape")
+    n = x.shape[-1]
+    _require(weight.dim() == 1 and weight.shape[0] == n and weight.is_contiguous(), "weight must be [n] contiguous")
+    x2 = x.reshape(-1, n)
+    r2 = residual.reshape(-1, n)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    if r2.stride(1) != 1:
+        r2 = r2.contiguous()
+    rows = x2.shape[0]
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    r_out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    lib = _capi.load()
+    st = lib.mops_hip_add_rms_forward(x2.data_ptr(), x2.stride(0) if rows > 1 else n, r2.data_ptr(),
+                                      r2.stride(0) if rows > 1 else n, weight.data_ptr(), y.data_ptr(),
+                                      r_out.data_ptr(), rows, n, float(eps), _stream(x))
+    _capi.check("mops_hip_add_rms_forward", st)
+    return y, r_out
+
+
+_workspaces: dict = {}
+
+
+def _decode_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Per-(device, stream) scratch for split-context partials; grown on demand, reused across calls
+    on the same stream (kernels on one stream run in order, so reuse cannot race)."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+@register_hip_op
+def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens=None,
+                            block_table=None, softmax_scale=None, causal=True, **kwargs) -> torch.Tensor:
+    """Paged decode attention, q [B, 1, Hq, D] -> [B, 1, Hq, D] (call form: nanovllm/layers/attention.py:40-42)."""
+    _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
+    _require(cache_seqlens is not None and block_table is not None, "cache_seqlens and block_table are required")
+    _require_cuda_bf16("q", q)
+    _require_cuda_bf16("k_cache", k_cache)
+    _require_cuda_bf16("v_cache", v_cache)
+    _require(q.dim() == 4 and q.shape[1] == 1, "q must be [batch, 1, heads, head_dim] (one query token per sequence)")
+    batch, _, hq, d = q.shape
+    _require(k_cache.dim() == 4 and k_cache.shape == v_cache.shape, "caches must be [blocks, block_size, kv_heads, dim]")
+    _require(k_cache.is_contiguous() and v_cache.is_contiguous(), "caches must be contiguous")
+    num_blocks, block_size, hkv, dk = k_cache.shape
+    _require(dk == d and hq % hkv == 0, "head_dim / head-count mismatch between q and the cache")
+    _require(q.stride(3) == 1 and q.stride(2) == d, "q heads must be contiguous")
+    _require(cache_seqlens.dtype == torch.int32 and cache_seqlens.is_cuda and cache_seqlens.is_contiguous()
+             and cache_seqlens.numel() == batch, "cache_seqlens must be a contiguous int32 GPU tensor of [batch]")
+    _require(block_table.dtype == torch.int32 and block_table.is_cuda and block_table.dim() == 2
+             and block_table.shape[0] == batch and block_table.stride(1) == 1,
+             "block_table must be an int32 GPU tensor [batch, max_blocks] with contiguous rows")
+    scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(d)
+    max_blocks = block_table.shape[1]
+    out = torch.empty((batch, 1, hq, d), dtype=q.dtype, device=q.device)
+    lib = _capi.load()
+    nbytes = lib.mops_hip_paged_decode_workspace_bytes(batch, hq, hkv, max_blocks, block_size)
+    ws = _decode_workspace(q.device, nbytes)
+    st = lib.mops_hip_attn_paged_decode_bf16(q.data_ptr(), q.stride(0) if batch > 1 else hq * d, k_cache.data_ptr(),
+                                             v_cache.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(),
+                                             block_table.stride(0) if batch > 1 else max_blocks, out.data_ptr(),
+                                             batch, hq, hkv, d, block_size, num_blocks, max_blocks, scale,
+                                             ws.data_ptr(), ws.numel(), _stream(q))
+    _capi.check("mops_hip_attn_paged_decode_bf16", st)
+    return out
+
+
+@register_hip_op
+def flash_attn_varlen_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, max_seqlen_q=None, cu_seqlens_q=None,
+                           max_seqlen_k=None, cu_seqlens_k=None, softmax_scale=None, causal=True, block_table=None,
+                           **kwargs) -> torch.Tensor:
+    """Varlen causal prefill attention over packed [T, H, D] tensors (call form: nanovllm/layers/attention.py:34-37)."""
+    _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
+    if block_table is not None:
+        raise NotImplementedError("prefix-cache prefill (block_table given) is not implemented by the hip backend")
+    _require(causal, "only causal attention is implemented")
+    _require(cu_seqlens_q is not None and max_seqlen_q is not None, "cu_seqlens_q and max_seqlen_q are required")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _require_cuda_bf16(name, t)
+        _require(t.dim() == 3 and t.stride(2) == 1 and t.stride(1) == t.shape[2], f"{name} must be [T, H, D] with contiguous heads")
+    total, hq, d = q.shape
+    _require(k.shape == v.shape and k.shape[0] == total and k.shape[2] == d, "k/v must be [T, Hkv, D] matching q")
+    hkv = k.shape[1]
+    _require(hq % hkv == 0, "query heads must be a multiple of kv heads")
+    _require(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_cuda and cu_seqlens_q.is_contiguous(),
+             "cu_seqlens_q must be a contiguous int32 GPU tensor")
+    if cu_seqlens_k is not None and cu_seqlens_k is not cu_seqlens_q:
+        _require(cu_seqlens_k.shape == cu_seqlens_q.shape, "cu_seqlens_k must match cu_seqlens_q (no prefix cache)")
+    batch = cu_seqlens_q.numel() - 1
+    scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(d)
+    out = torch.empty((total, hq, d), dtype=q.dtype, device=q.device)
+    lib = _capi.load()
+    ts = lambda t, h: t.stride(0) if total > 1 else h * d  # noqa: E731
+    st = lib.mops_hip_attn_varlen_causal_bf16(q.data_ptr(), ts(q, hq), k.data_ptr(), ts(k, hkv), v.data_ptr(),
+                                              ts(v, hkv), out.data_ptr(), hq * d, cu_seqlens_q.data_ptr(), batch,
+                                              total, int(max_seqlen_q), hq, hkv, d, scale, _stream(q))
+    _capi.check("mops_hip_attn_varlen_causal_bf16", st)
+    return out
+
+
+# ----------------------------------------------------------------------------------------------------
+# remaining registry names: library torch on the GPU, as in mops/torch/ops.py:5-7,32-54
+# ----------------------------------------------------------------------------------------------------
+
+@register_hip_op
+def linear(x, weight, bias=None):
+    return torch.nn.functional.linear(x, weight, bias)
+
+
+@register_hip_op
+def siluAndMul(x: torch.Tensor, y: torch.Tensor):
+    return torch.nn.functional.silu(x) * y
+
+
+@register_hip_op
+def sampler_forward(logits: torch.Tensor, temperatures: torch.Tensor):
+    logits = logits.float().div_(temperatures.unsqueeze(dim=1))
+    probs = torch.softmax(logits, dim=-1)
+    return torch.argmax(probs, dim=-1)
+
+
+@register_hip_op
+def apply_rotary_emb(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    x1, x2 = torch.chunk(x.float(), 2, dim=-1)
+    y1 = x1 * cos - x2 * sin
+    y2 = x2 * cos + x1 * sin
+    return torch.cat((y1, y2), dim=-1).to(x.dtype)
+
+
+@register_hip_op
+def softmax(x: torch.Tensor, dim: int = -1):
+    return torch.softmax(x, dim=dim)

@@ -1,0 +1,142 @@
+"""GPU parity for paged decode attention (flash_attn_with_kvcache) through the hip backend.
+
+Tolerance: max-abs 2e-2, mean-abs 2e-3 against the fp32 oracle (bf16 inputs/outputs, fp32 accumulate)."""
+import pytest
+import torch
+
+from helpers import assert_attention_close, assert_bit_exact
+from nano_vllm_ninetoothed_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(hip, d, gpu):
+    g = W.to_device(d, gpu)
+    return hip(g["q"], g["k_cache"], g["v_cache"], cache_seqlens=g["cache_seqlens"], block_table=g["block_table"],
+               softmax_scale=d["scale"], causal=True)
+
+
+def _ref(ref, d):
+    clean = dict(d)
+    return ref(d["q"], torch.nan_to_num(d["k_cache"]), torch.nan_to_num(d["v_cache"]), cache_seqlens=d["cache_seqlens"],
+               block_table=d["block_table"], softmax_scale=d["scale"], causal=True)
+
+
+@pytest.mark.parametrize("ctx,hq,hkv", [
+    ([1], 16, 8), ([31], 16, 8), ([32], 16, 8), ([33], 16, 8), ([255], 16, 8), ([256], 16, 8), ([257], 16, 8),
+    ([512, 513, 1, 1024, 300], 16, 8), ([700, 64, 2048, 257], 32, 8), ([4096, 3, 1000], 16, 8),
+    ([100, 200], 8, 8), ([640, 1300], 8, 1), ([900], 64, 4)])
+def test_decode_matches_oracle(gpu, ops, ctx, hq, hkv):
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs(ctx, hq=hq, hkv=hkv, seed=sum(ctx) + hq, poison_tail=True, extra_blocks=2)
+    got = _run(hip, d, gpu)
+    assert got.shape == (len(ctx), 1, hq, 128) and got.dtype == torch.bfloat16
+    assert_attention_close(got, _ref(ref, d), f"decode ctx={ctx} {hq}:{hkv}")
+
+
+def test_decode_batch_of_ragged_contexts(gpu, ops):
+    hip, ref = ops("flash_attn_with_kvcache")
+    ctx = W.random_seq_lens(48, 1, 4096, seed=2)
+    d = W.decode_inputs(ctx, seed=2, poison_tail=True)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), "ragged batch")
+
+
+def test_decode_zero_length_rows_are_zero_and_finite(gpu, ops):
+    """Graph-replay padding hands cache_seqlens == 0 rows (model_runner.py:202 of the reference)."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs([300, 1, 700], seed=4, poison_tail=True)
+    d["cache_seqlens"] = torch.tensor([300, 0, 700], dtype=torch.int32)
+    d["block_table"][1] = -1
+    got = _run(hip, d, gpu)
+    assert torch.isfinite(got.float()).all()
+    assert (got[1].float() == 0).all()
+    want = _ref(ref, d)
+    assert_attention_close(got[[0, 2]], want[[0, 2]], "non-empty rows")
+
+
+def test_decode_invariant_under_block_permutation(gpu, ops):
+    hip, _ = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs([1000, 257, 513], seed=6)
+    base = _run(hip, d, gpu)
+    nb = d["k_cache"].shape[0]
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(1))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(nb)
+    d2 = dict(d)
+    d2["k_cache"] = d["k_cache"][perm]
+    d2["v_cache"] = d["v_cache"][perm]
+    tbl = d["block_table"].clone()
+    mask = tbl >= 0
+    tbl[mask] = inv[tbl[mask].long()].to(torch.int32)
+    d2["block_table"] = tbl
+    assert_bit_exact(_run(hip, d2, gpu), base, "permuting blocks + table")
+
+
+def test_decode_equals_last_row_of_prefill(gpu, ops):
+    dec, _ = ops("flash_attn_with_kvcache")
+    pre, _ = ops("flash_attn_varlen_func")
+    L = 777
+    p = W.prefill_inputs([L], seed=8)
+    nb = (L + 255) // 256
+    kc = torch.zeros((nb, 256, 8, 128), dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    kc.view(-1, 8, 128)[:L] = p["k"]
+    vc.view(-1, 8, 128)[:L] = p["v"]
+    o_pre = pre(p["q"].to(gpu), p["k"].to(gpu), p["v"].to(gpu), max_seqlen_q=L, cu_seqlens_q=p["cu_seqlens"].to(gpu),
+                max_seqlen_k=L, cu_seqlens_k=p["cu_seqlens"].to(gpu), softmax_scale=p["scale"], causal=True, block_table=None)
+    o_dec = dec(p["q"][L - 1:L].unsqueeze(1).to(gpu), kc.to(gpu), vc.to(gpu),
+                cache_seqlens=torch.tensor([L], dtype=torch.int32, device=gpu),
+                block_table=torch.arange(nb, dtype=torch.int32, device=gpu).view(1, nb), softmax_scale=p["scale"], causal=True)
+    assert_attention_close(o_dec[0, 0], o_pre[L - 1], "decode vs last prefill row")
+
+
+def test_decode_single_token_returns_v_and_constant_v(gpu, ops):
+    hip, _ = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs([1, 600], seed=10)
+    d["v_cache"][d["block_table"][1, :3].long()] = 0.5      # constant V for sequence 1
+    got = _run(hip, d, gpu).cpu()
+    v0 = d["v_cache"][d["block_table"][0, 0].long(), 0]     # [8, 128]
+    assert_bit_exact(got[0, 0], v0.repeat_interleave(2, dim=0), "L=1 -> o = v")
+    assert (got[1].float() == 0.5).all(), "constant V -> o = V"
+
+
+def test_decode_wide_padded_table_and_strided_q(gpu, ops):
+    """block_table wider than needed (padded with -1) and q taken as a view of a [B, Hq*D + extra] buffer."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs([300, 900], seed=12, poison_tail=True)
+    wide = torch.full((2, 40), -1, dtype=torch.int32)
+    wide[:, :d["block_table"].shape[1]] = d["block_table"]
+    d["block_table"] = wide
+    want = _ref(ref, d)
+    g = W.to_device(d, gpu)
+    buf = torch.zeros((2, 16 * 128 + 2048), dtype=torch.bfloat16, device=gpu)
+    buf[:, :2048] = g["q"].view(2, -1)
+    qv = buf[:, :2048].view(2, 16, 128).unsqueeze(1)
+    got = hip(qv, g["k_cache"], g["v_cache"], cache_seqlens=g["cache_seqlens"], block_table=g["block_table"],
+              softmax_scale=d["scale"], causal=True)
+    assert_attention_close(got, want, "wide table / strided q")
+
+
+def test_decode_large_scores_stay_finite(gpu, ops):
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs([1500], seed=14, cache_std=6.0)
+    d["q"] = d["q"] * 4
+    got = _run(hip, d, gpu)
+    assert torch.isfinite(got.float()).all()
+    assert_attention_close(got, _ref(ref, d), "peaky softmax")
+
+
+@pytest.mark.parametrize("hq,hkv,lo,hi,bsz", [(16, 8, 512, 4096, 256)])
+def test_decode_full_size_properties(gpu, ops, hq, hkv, lo, hi, bsz):
+    """Benchmark-size run (256 sequences, 512..4096 context): checked on a sample of sequences against the
+    oracle, plus finiteness of everything and the convex-hull bound |o| <= max|v| of its context."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    ctx = W.random_seq_lens(bsz, lo, hi, seed=0)
+    d = W.decode_inputs(ctx, hq=hq, hkv=hkv, seed=0)
+    got = _run(hip, d, gpu).cpu()
+    assert torch.isfinite(got.float()).all()
+    assert got.float().abs().max() <= d["v_cache"].float().abs().max()
+    pick = [0, 1, 17, 100, 255, int(torch.tensor(ctx).argmax()), int(torch.tensor(ctx).argmin())]
+    sub = {"q": d["q"][pick], "k_cache": d["k_cache"], "v_cache": d["v_cache"], "cache_seqlens": d["cache_seqlens"][pick],
+           "block_table": d["block_table"][pick], "scale": d["scale"]}
+    assert_attention_close(got[pick], _ref(ref, sub), "sampled sequences of the full-size batch")

@@ -1,0 +1,123 @@
+"""GPU parity for varlen causal prefill attention (flash_attn_varlen_func) through the hip backend.
+
+Tolerance: max-abs 2e-2, mean-abs 2e-3 against the fp32 oracle (bf16 inputs/outputs, fp32 accumulate)."""
+import pytest
+import torch
+
+from helpers import assert_attention_close, assert_bit_exact
+from nano_vllm_ninetoothed_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(hip, d, gpu, **over):
+    g = W.to_device(d, gpu)
+    kw = dict(max_seqlen_q=d["max_seqlen"], cu_seqlens_q=g["cu_seqlens"], max_seqlen_k=d["max_seqlen"],
+              cu_seqlens_k=g["cu_seqlens"], softmax_scale=d["scale"], causal=True, block_table=None)
+    kw.update(over)
+    return hip(g["q"], g["k"], g["v"], **kw)
+
+
+def _ref(ref, d):
+    return ref(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"],
+               max_seqlen_k=d["max_seqlen"], cu_seqlens_k=d["cu_seqlens"], softmax_scale=d["scale"], causal=True)
+
+
+@pytest.mark.parametrize("lens,hq,hkv", [
+    ([256, 256], 16, 8), ([1], 16, 8), ([1, 1, 1], 16, 8), ([5], 16, 8), ([63, 64, 65], 16, 8),
+    ([127, 128, 129], 16, 8), ([300, 1, 77, 513], 16, 8), ([1000], 32, 8), ([200, 345], 8, 8),
+    ([130, 70], 8, 1), ([2048], 16, 8)])
+def test_prefill_matches_oracle(gpu, ops, lens, hq, hkv):
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs(lens, hq=hq, hkv=hkv, seed=sum(lens) + hq)
+    got = _run(hip, d, gpu)
+    assert got.shape == d["q"].shape and got.dtype == torch.bfloat16
+    assert_attention_close(got, _ref(ref, d), f"prefill lens={lens} {hq}:{hkv}")
+
+
+def test_prefill_v_is_strided_view_and_max_seqlen_is_only_a_bound(gpu, ops):
+    """q, k, v as nanovllm hands them: slices of one [T, 4096] qkv buffer (row stride 4096)."""
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([190, 333], seed=21)
+    T = 523
+    qkv = torch.cat([d["q"].view(T, -1), d["k"].view(T, -1), d["v"].view(T, -1)], dim=1).to(gpu)
+    q, k, v = qkv.split([2048, 1024, 1024], dim=-1)
+    cu = d["cu_seqlens"].to(gpu)
+    got = hip(q.view(T, 16, 128), k.view(T, 8, 128), v.view(T, 8, 128), max_seqlen_q=4096, cu_seqlens_q=cu,
+              max_seqlen_k=4096, cu_seqlens_k=cu, softmax_scale=d["scale"], causal=True, block_table=None)
+    assert got.is_contiguous()
+    assert_attention_close(got, _ref(ref, d), "strided qkv views")
+
+
+def test_prefill_sequences_do_not_leak_into_each_other(gpu, ops):
+    """Changing sequence 1 must not change sequence 0's output bits; NaN in a later sequence stays there."""
+    hip, _ = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([100, 150, 60], seed=23)
+    base = _run(hip, d, gpu).cpu()
+    d2 = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+    d2["k"][100:250] = float("nan")
+    d2["v"][100:250] = float("nan")
+    got = _run(hip, d2, gpu).cpu()
+    assert_bit_exact(got[:100], base[:100], "sequence 0")
+    assert_bit_exact(got[250:], base[250:], "sequence 2")
+
+
+def test_prefill_first_token_returns_v_and_constant_v(gpu, ops):
+    hip, _ = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([40, 300], seed=25)
+    d["v"][40:] = -1.25
+    got = _run(hip, d, gpu).cpu()
+    assert_bit_exact(got[0], d["v"][0].repeat_interleave(2, dim=0), "row 0 sees only key 0")
+    assert (got[40:].float() == -1.25).all()
+
+
+def test_prefill_empty_sequence_in_batch_and_no_tokens(gpu, ops):
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([70, 0, 130], seed=27)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), "batch with an empty sequence")
+    e = torch.empty((0, 16, 128), dtype=torch.bfloat16, device=gpu)
+    ek = torch.empty((0, 8, 128), dtype=torch.bfloat16, device=gpu)
+    cu = torch.zeros(1, dtype=torch.int32, device=gpu)
+    out = hip(e, ek, ek, max_seqlen_q=0, cu_seqlens_q=cu, max_seqlen_k=0, cu_seqlens_k=cu, softmax_scale=1.0, causal=True)
+    assert out.shape == (0, 16, 128)
+
+
+def test_prefill_rejects_prefix_cache_and_non_causal(gpu, ops):
+    hip, _ = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([32], seed=29)
+    with pytest.raises(NotImplementedError):
+        _run(hip, d, gpu, block_table=torch.zeros((1, 1), dtype=torch.int32, device=gpu))
+    with pytest.raises(ValueError):
+        _run(hip, d, gpu, causal=False)
+
+
+def test_prefill_warmup_shape(gpu, ops):
+    """The engine's warm-up batch: 4 sequences of 4096 tokens (model_runner.py:94-97 of the reference);
+    checked on sampled rows against the oracle."""
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([4096] * 4, seed=31)
+    got = _run(hip, d, gpu).cpu()
+    assert torch.isfinite(got.float()).all()
+    rows = [0, 1, 127, 128, 4095, 4096, 4096 + 2047, 3 * 4096 + 4095]
+    from oracle.bruteforce import attention_row  # fp64 definition, row by row
+    import numpy as np
+    for r in rows:
+        s, i = divmod(r, 4096)
+        lo = s * 4096
+        for h in (0, 15):
+            want = attention_row(d["q"][r, h].float().numpy(), d["k"][lo:lo + i + 1, h // 2].float().numpy(),
+                                 d["v"][lo:lo + i + 1, h // 2].float().numpy(), d["scale"]) if i < 300 else None
+            if want is not None:
+                assert np.abs(got[r, h].float().numpy() - want).max() <= 2e-2
+    sub = W.prefill_inputs([4096], seed=31)  # same generator stream -> same first sequence? not guaranteed; check via oracle on slice
+    one = {"q": d["q"][:4096], "k": d["k"][:4096], "v": d["v"][:4096], "cu_seqlens": torch.tensor([0, 4096], dtype=torch.int32),
+           "max_seqlen": 4096, "scale": d["scale"]}
+    assert_attention_close(got[:4096], _ref(ref, one), "first warm-up sequence")
+
+
+def test_prefill_full_size_config(gpu, ops):
+    """Benchmark-size batch: 16 sequences, lengths uniform in [128, 2048]; whole output vs the oracle."""
+    hip, ref = ops("flash_attn_varlen_func")
+    lens = W.random_seq_lens(16, 128, 2048, seed=0)
+    d = W.prefill_inputs(lens, seed=0)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), "cfg2")
