@@ -1,0 +1,296 @@
+#!/usr/bin/env python3
+"""Benchmark of the mops `hip` backend on one MI355X.
+
+Default run = the headline workload: paged decode attention at Qwen3-0.6B shape (256 sequences, one
+query token each, 16 q heads / 8 kv heads, head_dim 128, context uniform in [512, 4096], block 256).
+A step is one flash_attn_with_kvcache call over the whole batch, KV cache resident in HBM.
+`--op` selects another operator of the hot path (same JSON format, its own metric):
+  decode (default) | decode8b | prefill | store | add_rms | rms | embedding
+
+Prints ONE JSON line on stdout.  `roofline` is computed from HIP-event time of the op on its launch
+stream; `cpu_baseline` times the CPU restatement of the reference's torch backend (oracle/) on a
+bounded sample of the same workload on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--op", default="decode",
+                    choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); the hot path has no "
+              "cross-GPU exchange, see DESIGN.md for how it shards.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from nano_vllm_ninetoothed_amd import _capi, mops
+    from nano_vllm_ninetoothed_amd import workloads as W
+    _capi.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+
+    def randn_bf16(shape, std=1.0):
+        return (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std).to(torch.bfloat16) \
+            if torch.Size(shape).numel() < (1 << 28) else _big_randn(shape, std)
+
+    def _big_randn(shape, std):
+        out = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+        flat = out.view(-1)
+        step = 1 << 27
+        for i in range(0, flat.numel(), step):
+            n = min(step, flat.numel() - i)
+            flat[i:i + n] = (torch.randn(n, generator=g, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+        return out
+
+    cpu_fn = None      # () -> (seconds, description, units_done)  on a bounded sample
+    bound = "hbm"
+    dtype = "bf16"
+
+    # ------------------------------------------------------------------ workloads
+    if args.op in ("decode", "decode8b"):
+        if args.op == "decode":
+            bsz, hq, hkv, lo, hi, name = 256, 16, 8, 512, 4096, "cfg3 paged decode, Qwen3-0.6B shape"
+        else:
+            bsz, hq, hkv, lo, hi, name = 512, 32, 8, 1024, 8192, "cfg4 paged decode, Qwen3-8B shape"
+        ctx = W.random_seq_lens(bsz, lo, hi, seed=args.seed)
+        blocks_per_seq = [(c + W.BLOCK_SIZE - 1) // W.BLOCK_SIZE for c in ctx]
+        nblk = sum(blocks_per_seq)
+        max_blocks = max(blocks_per_seq)
+        perm = torch.randperm(nblk, generator=torch.Generator().manual_seed(args.seed)).to(torch.int32)
+        table = torch.full((bsz, max_blocks), -1, dtype=torch.int32)
+        pos = 0
+        for b, nb in enumerate(blocks_per_seq):
+            table[b, :nb] = perm[pos:pos + nb]
+            pos += nb
+        n_copies = 2 if args.op == "decode" else 1   # rotate KV buffers so no step re-reads warm lines
+        caches = [(randn_bf16((nblk, W.BLOCK_SIZE, hkv, W.HEAD_DIM)), randn_bf16((nblk, W.BLOCK_SIZE, hkv, W.HEAD_DIM)))
+                  for _ in range(n_copies)]
+        q = randn_bf16((bsz, 1, hq, W.HEAD_DIM))
+        lens_g = torch.tensor(ctx, dtype=torch.int32, device=dev)
+        table_g = table.to(dev)
+        scale = W.HEAD_DIM ** -0.5
+        op = mops.flash_attn_with_kvcache
+
+        def step(i):
+            kc, vc = caches[i % n_copies]
+            return op(q, kc, vc, cache_seqlens=lens_g, block_table=table_g, softmax_scale=scale, causal=True)
+
+        work = W.decode_bytes(ctx, hq, hkv, max_blocks)      # algorithmic bytes per step
+        metric, unit = "paged_decode_attn_GBps", "GB/s"
+        config = {"workload": name, "batch": bsz, "q_heads": hq, "kv_heads": hkv, "head_dim": W.HEAD_DIM,
+                  "block_size": W.BLOCK_SIZE, "context": f"uniform[{lo},{hi}] seed {args.seed}",
+                  "context_tokens": sum(ctx), "kv_buffers_rotated": n_copies}
+        kernel_name = "paged_decode_kernel (+ paged_decode_combine_kernel)"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("flash_attn_with_kvcache", "torch")
+            n = 32
+            sub_tbl = table[:n]
+            used = sub_tbl[sub_tbl >= 0].long()
+            remap = torch.full((nblk,), -1, dtype=torch.int32)
+            remap[used] = torch.arange(len(used), dtype=torch.int32)
+            tbl = torch.where(sub_tbl >= 0, remap[sub_tbl.clamp(min=0).long()], sub_tbl)
+            kc = caches[0][0][used.to(dev)].cpu()
+            vc = caches[0][1][used.to(dev)].cpu()
+            qc = q[:n].cpu()
+            lens = torch.tensor(ctx[:n], dtype=torch.int32)
+            ref(qc, kc, vc, cache_seqlens=lens, block_table=tbl, softmax_scale=scale)
+            ts = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                ref(qc, kc, vc, cache_seqlens=lens, block_table=tbl, softmax_scale=scale)
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[1], f"first {n} of {bsz} sequences, median of 3", W.decode_bytes(ctx[:n], hq, hkv, max_blocks)
+
+    elif args.op == "prefill":
+        lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
+        d = W.to_device(W.prefill_inputs(lens, seed=args.seed), dev)
+        op = mops.flash_attn_varlen_func
+
+        def step(i):
+            return op(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"],
+                      max_seqlen_k=d["max_seqlen"], cu_seqlens_k=d["cu_seqlens"], softmax_scale=d["scale"], causal=True)
+
+        work = W.prefill_flops(lens, 16)
+        bound = "mfma"
+        metric, unit = "varlen_prefill_attn_TFLOPs", "TFLOP/s"
+        config = {"workload": "cfg2 varlen causal prefill, Qwen3-0.6B shape", "batch": 16, "q_heads": 16, "kv_heads": 8,
+                  "head_dim": 128, "seq_lens": f"uniform[128,2048] seed {args.seed}", "total_tokens": sum(lens)}
+        kernel_name = "varlen_prefill_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("flash_attn_varlen_func", "torch")
+            c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+            ts = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                ref(c["q"], c["k"], c["v"], max_seqlen_q=c["max_seqlen"], cu_seqlens_q=c["cu_seqlens"], softmax_scale=c["scale"])
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[1], "whole batch, median of 3", work
+
+    elif args.op == "store":
+        lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
+        T = sum(lens)
+        n_copies = 4
+        sets = []
+        for i in range(n_copies):
+            s = W.to_device(W.store_inputs(T, seed=args.seed + i, v_row_stride=4096), dev)
+            wide = s["value"]
+            s["value"] = wide
+            s["kc"] = torch.zeros((s["num_blocks"], 256, 8, 128), dtype=torch.bfloat16, device=dev)
+            s["vc"] = torch.zeros_like(s["kc"])
+            sets.append(s)
+        op = mops.store_kvcache
+
+        def step(i):
+            s = sets[i % n_copies]
+            return op(s["key"], s["value"], s["kc"], s["vc"], s["slot_mapping"])
+
+        work = float(2 * T * 1024 * 2 * 2 + 4 * T)
+        metric, unit = "store_kvcache_GBps", "GB/s"
+        config = {"workload": "cfg2 store_kvcache", "tokens": T, "row_bytes": 2048, "buffers_rotated": n_copies}
+        kernel_name = "store_kvcache_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("store_kvcache", "torch")
+            s = sets[0]
+            k, v, kc, vc, sl = (s[x].cpu() for x in ("key", "value", "kc", "vc", "slot_mapping"))
+            ts = []
+            for _ in range(5):
+                t0 = time.perf_counter()
+                ref(k, v, kc, vc, sl)
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[2], "whole batch, median of 5", work
+
+    elif args.op in ("add_rms", "rms"):
+        rows, hidden = 512, 4096
+        n_copies = 24   # 24 x 16.8 MB > 256 MB of last-level cache
+        sets = [W.to_device(W.rms_inputs(rows, hidden, seed=args.seed + i, with_residual=True), dev) for i in range(n_copies)]
+        if args.op == "add_rms":
+            op = mops.add_rms_forward
+
+            def step(i):
+                s = sets[i % n_copies]
+                return op(s["x"], s["residual"], s["weight"], s["eps"])
+            work = float(4 * rows * hidden * 2 + hidden * 2)
+        else:
+            op = mops.rms_forward
+
+            def step(i):
+                s = sets[i % n_copies]
+                return op(s["x"], s["weight"], s["eps"])
+            work = float(2 * rows * hidden * 2 + hidden * 2)
+        metric, unit = f"{args.op}_forward_GBps", "GB/s"
+        config = {"workload": f"cfg4 {args.op}_forward", "rows": rows, "hidden": hidden, "buffers_rotated": n_copies}
+        kernel_name = "rmsnorm_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op(f"{args.op}_forward", "torch")
+            s = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in sets[0].items()}
+            a = (s["x"], s["residual"], s["weight"], s["eps"]) if args.op == "add_rms" else (s["x"], s["weight"], s["eps"])
+            ts = []
+            for _ in range(7):
+                t0 = time.perf_counter()
+                ref(*a)
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[3], "whole batch, median of 7", work
+
+    else:  # embedding
+        vocab, hidden, n_ids = 151936, 4096, 512
+        weight = _big_randn((vocab, hidden), 0.02)
+        ids = [torch.randint(0, vocab, (n_ids,), generator=g, device=dev, dtype=torch.int32) for _ in range(64)]
+        op = mops.embedding
+
+        def step(i):
+            return op(ids[i % len(ids)], weight)
+
+        work = float(2 * n_ids * hidden * 2 + n_ids * 4)
+        metric, unit = "embedding_GBps", "GB/s"
+        config = {"workload": "cfg4 embedding", "vocab": vocab, "hidden": hidden, "ids": n_ids, "id_sets_rotated": len(ids)}
+        kernel_name = "embedding_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("embedding", "torch")
+            w, x = weight.cpu(), ids[0].cpu()
+            ts = []
+            for _ in range(7):
+                t0 = time.perf_counter()
+                ref(x, w)
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[3], "whole batch, median of 7", work
+
+    # ------------------------------------------------------------------ timed region
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(args.steps):
+        step(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per_step_ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)]
+    ev_ms = sum(per_step_ms) / len(per_step_ms)
+    ms_per_step = wall * 1e3 / args.steps
+
+    if bound == "hbm":
+        value = work / (ms_per_step * 1e-3) / 1e9
+        achieved = work / (ev_ms * 1e-3) / 1e9
+        peak, runit = HBM_PEAK_GBPS, "GB/s"
+    else:
+        value = work / (ms_per_step * 1e-3) / 1e12
+        achieved = work / (ev_ms * 1e-3) / 1e12
+        peak, runit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+
+    out = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic", "config": config,
+        "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": runit,
+                     "frac": round(achieved / peak, 4), "traffic": None, "kernel": kernel_name,
+                     "algorithmic_work_per_launch": work, "event_ms_per_launch": round(ev_ms, 5),
+                     "event_ms_min": round(min(per_step_ms), 5)},
+    }
+    if not args.no_cpu_baseline and cpu_fn is not None:
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        secs, sample, units = cpu_fn()
+        cval = units / secs / (1e9 if bound == "hbm" else 1e12)
+        out["cpu_baseline"] = {"value": round(cval, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": sample, "seconds": round(secs, 4)}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

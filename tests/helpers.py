@@ -47,3 +47,41 @@ def assert_attention_close(got: torch.Tensor, want: torch.Tensor, what: str = ""
     diff = (g - w).abs()
     assert diff.max().item() <= ATTN_MAX_ABS, f"{what}: max-abs {diff.max().item():.4g} > {ATTN_MAX_ABS}"
     assert diff.mean().item() <= ATTN_MEAN_ABS, f"{what}: mean-abs {diff.mean().item():.4g} > {ATTN_MEAN_ABS}"
+
+
+def _step_bf16(t: torch.Tensor, direction: int) -> torch.Tensor:
+    """Neighbouring representable bf16 in value order: direction +1 = next larger, -1 = next smaller."""
+    bits = t.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
+    neg = bits >= 0x8000
+    mag = bits & 0x7FFF
+    # value order: positive numbers grow with mag, negative shrink
+    delta = torch.where(neg, torch.full_like(mag, -direction), torch.full_like(mag, direction))
+    new_mag = mag + delta
+    flip = new_mag < 0                       # crossed zero
+    new_mag = torch.where(flip, torch.ones_like(new_mag), new_mag)
+    new_neg = torch.where(flip, ~neg, neg)
+    out = (new_mag | (new_neg.to(torch.int32) << 15)).to(torch.int32)
+    out = torch.where(out >= 0x8000, out - 0x10000, out).to(torch.int16)
+    return out.view(torch.bfloat16)
+
+
+def assert_rms_parity(got: torch.Tensor, normed_ref: torch.Tensor, weight: torch.Tensor, want: torch.Tensor, what: str = ""):
+    """RMSNorm has two bf16 roundings: bf16(x * rstd), then bf16(that * w).  The row statistic is an fp32
+    sum whose last bit depends on summation order, which can move the FIRST rounding by one bf16 step.
+    Accepted: the output equals, bit for bit, what the reference's second stage produces from a
+    normalised value at most 1 bf16 ulp from the reference's (normed_ref); and at least 99.9 % of the
+    elements equal the reference output exactly."""
+    got = got.cpu()
+    assert got.shape == want.shape and got.dtype == torch.bfloat16
+    assert torch.isfinite(got.float()).all(), f"{what}: non-finite"
+    cands = [normed_ref * weight, _step_bf16(normed_ref, +1) * weight, _step_bf16(normed_ref, -1) * weight]
+    ok = torch.zeros(got.shape, dtype=torch.bool)
+    gb = got.contiguous().view(torch.int16)
+    for c in cands:
+        ok |= gb == c.contiguous().view(torch.int16)
+    # -0.0 vs +0.0 are the same value
+    ok |= (got.float() == 0) & (want.float() == 0)
+    bad = int((~ok).sum())
+    assert bad == 0, f"{what}: {bad} elements are not reachable from a normalised value within 1 bf16 ulp"
+    exact = (gb == want.contiguous().view(torch.int16)).float().mean().item()
+    assert exact >= 0.999, f"{what}: only {exact:.5f} of the elements equal the reference bit for bit"

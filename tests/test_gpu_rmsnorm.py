@@ -1,12 +1,21 @@
-"""GPU parity for rms_forward / add_rms_forward: within 1 bf16 ulp of the oracle on the same inputs."""
+"""GPU parity for rms_forward / add_rms_forward against the oracle on the same inputs.
+
+Tolerance: 1 bf16 ulp at the normalisation rounding (helpers.assert_rms_parity): the output must be
+bit-identical to the reference's second stage applied to a normalised value within 1 bf16 ulp of the
+reference's, and >= 99.9 % of all elements must equal the reference output exactly."""
 import pytest
 import torch
 
-from helpers import assert_bit_exact, assert_within_one_ulp, ulp_distance_bf16
+from helpers import assert_bit_exact, assert_rms_parity
 from nano_vllm_ninetoothed_amd import workloads as W
 
 pytestmark = pytest.mark.gpu
-ULP_TOL = 1  # bf16 units in the last place
+
+
+def _normed(x, eps, residual=None):
+    """The reference's value after its first rounding (mops/torch/ops.py:11-15 / 21-29)."""
+    s = x.float() if residual is None else x.float() + residual.float()
+    return (s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps)).to(torch.bfloat16)
 
 
 @pytest.mark.parametrize("rows,hidden", [(512, 1024), (512, 4096), (1, 1024), (7, 128), (333, 128), (65, 2048),
@@ -20,9 +29,7 @@ def test_rms_forward_2d(gpu, ops, rows, hidden):
     got = hip(x_g, d["weight"].to(gpu), d["eps"])
     assert got.data_ptr() != x_g.data_ptr()
     assert_bit_exact(x_g, keep, "input left intact")
-    assert_within_one_ulp(got, want, f"rms_forward {rows}x{hidden}")
-    frac_exact = (ulp_distance_bf16(got, want) == 0).float().mean().item()
-    assert frac_exact > 0.99, f"only {frac_exact:.4f} of elements bit-equal"
+    assert_rms_parity(got, _normed(d["x"], d["eps"]), d["weight"], want, f"rms_forward {rows}x{hidden}")
 
 
 def test_rms_forward_strided_qk_views(gpu, ops):
@@ -40,7 +47,7 @@ def test_rms_forward_strided_qk_views(gpu, ops):
         assert not gv.is_contiguous()
         got = hip(gv, w.to(gpu), 1e-6)
         assert got.shape == (T, heads, 128) and got.is_contiguous()
-        assert_within_one_ulp(got, ref(cv, w, 1e-6), f"{name}_norm")
+        assert_rms_parity(got, _normed(cv, 1e-6), w, ref(cv, w, 1e-6), f"{name}_norm")
     assert_bit_exact(qkv_g, qkv, "qkv buffer untouched")
 
 
@@ -50,7 +57,7 @@ def test_rms_forward_3d_contiguous_and_empty(gpu, ops):
     x3 = d["x"].view(2, 12, 1024)
     got = hip(x3.to(gpu), d["weight"].to(gpu), 1e-6)
     assert got.shape == (2, 12, 1024)
-    assert_within_one_ulp(got, ref(x3, d["weight"], 1e-6), "3-D")
+    assert_rms_parity(got, _normed(x3, 1e-6), d["weight"], ref(x3, d["weight"], 1e-6), "3-D")
     e = hip(torch.empty((0, 1024), dtype=torch.bfloat16, device=gpu), d["weight"].to(gpu), 1e-6)
     assert e.shape == (0, 1024)
 
@@ -63,7 +70,7 @@ def test_add_rms_forward(gpu, ops, rows, hidden):
     x_g, r_g = d["x"].to(gpu), d["residual"].to(gpu)
     got_y, got_r = hip(x_g, r_g, d["weight"].to(gpu), d["eps"])
     assert_bit_exact(got_r, want_r, "residual output (a single fp32 add, rounded once)")
-    assert_within_one_ulp(got_y, want_y, f"add_rms_forward {rows}x{hidden}")
+    assert_rms_parity(got_y, _normed(d["x"], d["eps"], d["residual"]), d["weight"], want_y, f"add_rms_forward {rows}x{hidden}")
     assert_bit_exact(x_g, d["x"], "x untouched")
     assert_bit_exact(r_g, d["residual"], "residual input untouched")
 

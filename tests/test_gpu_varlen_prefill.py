@@ -109,7 +109,6 @@ def test_prefill_warmup_shape(gpu, ops):
                                  d["v"][lo:lo + i + 1, h // 2].float().numpy(), d["scale"]) if i < 300 else None
             if want is not None:
                 assert np.abs(got[r, h].float().numpy() - want).max() <= 2e-2
-    sub = W.prefill_inputs([4096], seed=31)  # same generator stream -> same first sequence? not guaranteed; check via oracle on slice
     one = {"q": d["q"][:4096], "k": d["k"][:4096], "v": d["v"][:4096], "cu_seqlens": torch.tensor([0, 4096], dtype=torch.int32),
            "max_seqlen": 4096, "scale": d["scale"]}
     assert_attention_close(got[:4096], _ref(ref, one), "first warm-up sequence")

@@ -1,0 +1,196 @@
+"""Pins the parity oracle (oracle/mops_torch.py) without a GPU: every check here is something other than a
+second copy of the oracle's own formula — closed forms in fp64, loop-level brute force on tiny inputs,
+library routines the ops reduce to, and invariants of the mathematics.  The reference ships no golden
+vectors or tests for these ops, so these checks are what stands behind "the oracle is right"."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bit_exact, ulp_distance_bf16
+from nano_vllm_ninetoothed_amd import workloads as W
+from oracle import bruteforce as BF
+
+
+@pytest.fixture(scope="module")
+def O():
+    import oracle.mops_torch as m
+    return m
+
+
+def to_bf16_from_f64(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(a).to(torch.float32).to(torch.bfloat16)
+
+
+# ------------------------------------------------------------------------------------------ norms
+
+@pytest.mark.parametrize("rows,hidden", [(16, 128), (9, 1024), (4, 4096)])
+def test_rms_forward_against_fp64_closed_form(O, rows, hidden):
+    d = W.rms_inputs(rows, hidden, seed=hidden)
+    got = O.rms_forward(d["x"], d["weight"], d["eps"])
+    exact = BF.rms(d["x"].float().numpy(), d["weight"].float().numpy(), d["eps"])
+    # two roundings: each at most half a bf16 step (2^-8 relative), the first scaled by |w|
+    err = np.abs(got.float().numpy().astype(np.float64) - exact)
+    bound = np.abs(exact) * (2.0 ** -8) * 2 + 1e-30
+    assert (err <= bound).all()
+    assert ulp_distance_bf16(got, to_bf16_from_f64(exact)).max() <= 2
+
+
+def test_rms_forward_special_rows(O):
+    w = torch.tensor([1.0, 0.5, -2.0, 1.5] * 32, dtype=torch.bfloat16)
+    zero = O.rms_forward(torch.zeros((1, 128), dtype=torch.bfloat16), w, 1e-6)
+    assert (zero.float() == 0).all()
+    c = 3.0
+    const = O.rms_forward(torch.full((1, 128), c, dtype=torch.bfloat16), w, 1e-6)
+    one = torch.tensor(1.0 / math.sqrt(1.0 + 1e-6 / (c * c)), dtype=torch.float32).to(torch.bfloat16)
+    assert_bit_exact(const[0], (one * w), "constant row -> sign(x) * w (after rounding 1/sqrt(1+eps/x^2))")
+    neg = O.rms_forward(torch.full((1, 128), -c, dtype=torch.bfloat16), w, 1e-6)
+    assert_bit_exact(neg[0], (-one * w), "negative constant row")
+    # scale invariance up to eps: rms(2x) == rms(x) when eps is negligible (powers of two are exact)
+    d = W.rms_inputs(8, 1024, seed=2)
+    a = O.rms_forward(d["x"], d["weight"], 0.0)
+    b = O.rms_forward(d["x"] * 2, d["weight"], 0.0)
+    assert_bit_exact(a, b, "scale invariance")
+    x3 = d["x"].view(2, 4, 1024)
+    assert_bit_exact(O.rms_forward(x3, d["weight"], 1e-6).view(8, 1024), O.rms_forward(d["x"], d["weight"], 1e-6), "3-D == 2-D")
+    assert O.rms_forward(d["x"], d["weight"], 1e-6).dtype == torch.bfloat16
+
+
+def test_add_rms_forward_reductions(O):
+    d = W.rms_inputs(12, 1024, seed=3, with_residual=True)
+    y0, r0 = O.add_rms_forward(d["x"], torch.zeros_like(d["x"]), d["weight"], d["eps"])
+    assert_bit_exact(y0, O.rms_forward(d["x"], d["weight"], d["eps"]), "zero residual -> rms_forward")
+    assert_bit_exact(r0, d["x"], "zero residual -> residual out is x")
+    y, r = O.add_rms_forward(d["x"], d["residual"], d["weight"], d["eps"])
+    assert_bit_exact(r, (d["x"].float() + d["residual"].float()).to(torch.bfloat16), "residual = rounded fp32 sum")
+    y2, r2 = O.add_rms_forward(d["residual"], d["x"], d["weight"], d["eps"])
+    assert_bit_exact(y, y2, "commutes in (x, residual)")
+    exact = BF.rms(d["x"].float().numpy().astype(np.float64) + d["residual"].float().numpy(), d["weight"].float().numpy(), d["eps"])
+    assert ulp_distance_bf16(y, to_bf16_from_f64(exact)).max() <= 2
+    # the statistic uses the UNROUNDED sum: normalising the rounded residual instead must differ somewhere
+    y_wrong = O.rms_forward(r, d["weight"], d["eps"])
+    assert not torch.equal(y_wrong.view(torch.int16), y.view(torch.int16))
+    before = d["x"].clone()
+    O.add_rms_forward(d["x"], d["residual"], d["weight"], d["eps"])
+    assert_bit_exact(d["x"], before, "inputs not mutated")
+
+
+# ------------------------------------------------------------------------------------------ copies
+
+def test_embedding_is_f_embedding(O):
+    d = W.embedding_inputs(200, 1000, 256, seed=1, id_dtype=torch.int64)
+    assert_bit_exact(O.embedding(d["ids"], d["weight"]), torch.nn.functional.embedding(d["ids"], d["weight"]), "F.embedding")
+    d32 = W.embedding_inputs(50, 1000, 256, seed=1, id_dtype=torch.int32)
+    assert_bit_exact(O.embedding(d32["ids"], d32["weight"]), d32["weight"].index_select(0, d32["ids"].long()), "int32 ids")
+    assert O.embedding(d["ids"].view(10, 20), d["weight"]).shape == (10, 20, 256)
+
+
+def test_store_kvcache_is_index_copy(O):
+    d = W.store_inputs(300, seed=7, v_row_stride=4096)
+    assert d["value"].stride(0) == 4096
+    kc = torch.full((d["num_blocks"], 256, 8, 128), -7.0, dtype=torch.bfloat16)
+    vc = torch.full_like(kc, 9.0)
+    slots = d["slot_mapping"].clone()
+    slots[5] = -1
+    slots[100] = -1
+    assert O.store_kvcache(d["key"], d["value"], kc, vc, slots) is None
+    keep = slots != -1
+    want_k = torch.full((d["num_blocks"] * 256, 1024), -7.0, dtype=torch.bfloat16)
+    want_k.index_copy_(0, slots[keep].long(), d["key"].reshape(300, 1024)[keep])
+    want_v = torch.full((d["num_blocks"] * 256, 1024), 9.0, dtype=torch.bfloat16)
+    want_v.index_copy_(0, slots[keep].long(), d["value"].reshape(300, 1024)[keep])
+    assert_bit_exact(kc.view(-1, 1024), want_k, "k_cache")
+    assert_bit_exact(vc.view(-1, 1024), want_v, "v_cache")
+    assert int((kc.view(-1, 1024)[:, 0] != -7.0).sum()) == 298
+    with pytest.raises(AssertionError):
+        O.store_kvcache(d["key"], d["value"], kc, vc, slots[:-1])
+    with pytest.raises(AssertionError):
+        O.store_kvcache(d["key"].transpose(1, 2), d["value"], kc, vc, slots)
+
+
+# ------------------------------------------------------------------------------------------ attention
+
+def _varlen(O, d, **kw):
+    return O.flash_attn_varlen_func(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"],
+                                    max_seqlen_k=d["max_seqlen"], cu_seqlens_k=d["cu_seqlens"], softmax_scale=d["scale"],
+                                    causal=True, block_table=None, **kw)
+
+
+@pytest.mark.parametrize("lens,hq,hkv", [([5, 1, 9], 4, 2), ([7], 8, 2), ([3, 4], 2, 2), ([6, 2], 4, 1)])
+def test_varlen_against_fp64_brute_force(O, lens, hq, hkv):
+    d = W.prefill_inputs(lens, hq=hq, hkv=hkv, seed=sum(lens) + hq)
+    got = _varlen(O, d).float().numpy()
+    want = BF.varlen_causal(d["q"].float().numpy(), d["k"].float().numpy(), d["v"].float().numpy(),
+                            d["cu_seqlens"].tolist(), d["scale"])
+    # only the final bf16 rounding separates fp32-accumulated attention from the fp64 definition
+    assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -8 + 1e-6
+
+
+def test_varlen_against_library_sdpa(O):
+    d = W.prefill_inputs([33, 70, 1], hq=16, hkv=8, seed=5)
+    got = _varlen(O, d)
+    cu = d["cu_seqlens"].tolist()
+    for s in range(3):
+        q, k, v = (d[n][cu[s]:cu[s + 1]].float().transpose(0, 1).unsqueeze(0) for n in ("q", "k", "v"))
+        want = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=d["scale"], enable_gqa=True)
+        want = want[0].transpose(0, 1)
+        assert (got[cu[s]:cu[s + 1]].float() - want).abs().max() <= 2e-2 / 2
+
+
+def test_varlen_invariants(O):
+    d = W.prefill_inputs([40, 25], seed=6)
+    base = _varlen(O, d)
+    assert_bit_exact(base[0], d["v"][0].repeat_interleave(2, dim=0), "first token of a sequence -> o = v (head h uses kv head h // 2)")
+    assert_bit_exact(base[40], d["v"][40].repeat_interleave(2, dim=0), "first token of the second sequence")
+    d2 = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+    d2["k"][40:] = 100.0
+    d2["v"][40:] = -3.0
+    got2 = _varlen(O, d2)
+    assert_bit_exact(got2[:40], base[:40], "sequence 0 independent of sequence 1")
+    assert (got2[40:].float() == -3.0).all(), "constant V -> o = V"
+    d3 = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+    d3["k"][30:40] = 50.0     # future keys of row 29 inside its own sequence
+    got3 = _varlen(O, d3)
+    assert_bit_exact(got3[:30], base[:30], "causality: rows < 30 never see keys >= 30")
+    default_scale = O.flash_attn_varlen_func(d["q"], d["k"], d["v"], cu_seqlens_q=d["cu_seqlens"], max_seqlen_q=40)
+    assert_bit_exact(default_scale, base, "default scale is 1/sqrt(head_dim)")
+
+
+def _decode(O, d):
+    return O.flash_attn_with_kvcache(d["q"], d["k_cache"], d["v_cache"], cache_seqlens=d["cache_seqlens"],
+                                     block_table=d["block_table"], softmax_scale=d["scale"], causal=True)
+
+
+@pytest.mark.parametrize("ctx,hq,hkv", [([3, 300], 4, 2), ([257], 2, 1), ([1, 256], 4, 4)])
+def test_decode_against_fp64_brute_force(O, ctx, hq, hkv):
+    d = W.decode_inputs(ctx, hq=hq, hkv=hkv, seed=sum(ctx))
+    got = _decode(O, d)[:, 0].float().numpy()
+    want = BF.paged_decode(d["q"][:, 0].float().numpy(), d["k_cache"].float().numpy(), d["v_cache"].float().numpy(),
+                           d["ctx_lens"], d["block_table"].tolist(), d["scale"])
+    assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -8 + 1e-6
+
+
+def test_decode_invariants(O):
+    L = 300
+    p = W.prefill_inputs([L], seed=8)
+    nb = 2
+    order = [1, 0]  # token t lives in block order[t // 256]
+    kc = torch.full((nb, 256, 8, 128), float("nan"), dtype=torch.bfloat16)
+    vc = torch.full_like(kc, float("nan"))
+    for t0 in range(0, L, 256):
+        n = min(256, L - t0)
+        kc[order[t0 // 256], :n] = p["k"][t0:t0 + n]
+        vc[order[t0 // 256], :n] = p["v"][t0:t0 + n]
+    d = {"q": p["q"][L - 1:L].unsqueeze(1), "k_cache": kc, "v_cache": vc, "cache_seqlens": torch.tensor([L], dtype=torch.int32),
+         "block_table": torch.tensor([order + [-1, -1]], dtype=torch.int32), "scale": p["scale"]}
+    got = _decode(O, d)
+    assert torch.isfinite(got.float()).all(), "NaN sentinels beyond cache_seqlens / -1 columns never reach the output"
+    pre = _varlen(O, p)
+    # same mathematics through differently shaped fp32 matmuls: equal up to the final bf16 rounding
+    assert ulp_distance_bf16(got[0, 0], pre[L - 1]).max() <= 1, "decode == last row of causal prefill over the same K/V"
+    assert got.shape == (1, 1, 16, 128)
+    d0 = dict(d, cache_seqlens=torch.tensor([0], dtype=torch.int32))
+    assert (_decode(O, d0).float() == 0).all(), "empty context -> zeros"
+    d1 = dict(d, cache_seqlens=torch.tensor([1], dtype=torch.int32))
+    assert_bit_exact(_decode(O, d1)[0, 0], vc[1, 0].repeat_interleave(2, dim=0), "one cached token -> o = v")
