@@ -6,10 +6,12 @@ fallback behind these functions.  Signatures mirror include/mops_hip.h one to on
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmops_hip.so"
+# MOPS_HIP_LIB points at another build of the same ABI (kernel tuning experiments)
+LIB_PATH = Path(os.environ.get("MOPS_HIP_LIB") or Path(__file__).resolve().parent / "lib" / "libmops_hip.so")
 
 # name -> (restype, argtypes); the exported surface declared in include/mops_hip.h
 SIGNATURES = {

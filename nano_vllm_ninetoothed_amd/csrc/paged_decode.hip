@@ -1,17 +1,28 @@
 // Paged decode attention for gfx950: one query token per sequence against the block-table-addressed
 // KV cache (layout [num_blocks, block_size, hkv, 128] bf16).  HBM-bandwidth bound: every K/V byte of
-// the live context is read exactly once, 16 bytes per lane, 256 contiguous bytes per token row.
+// the live context is read exactly once, 16 bytes per lane, 256 contiguous bytes per token and head.
 //
-// Work decomposition
-//   unit  = (chunk c, sequence b, kv head g): the tokens [c*chunk, (c+1)*chunk) of sequence b for one
-//           kv head, served for ALL hq/hkv query heads of that group from one read of K and V.
-//   one unit = one 64-lane workgroup (a single wave64): no workgroup barriers, the wave owns a private
-//           16 KiB LDS tile.  Units are numbered chunk-major so the units that fall beyond a
-//           sequence's length (they exit at once) collect at the end of the launch.
-//   stage = 32 consecutive tokens of the unit (inside one cache block): 8 KiB of K + 8 KiB of V.
-//           Stage i+1 is in flight from HBM into registers while stage i is consumed out of LDS.
+// Work is split "flat": the 32-token stages of all sequences are laid end to end and cut into ncols
+// equal runs, one per column of workgroups, so every column streams the same number of bytes no
+// matter how ragged the context lengths are.  A run may start in the middle of a sequence and may
+// cover several short ones; each (column, sequence) intersection is a piece.
 //
-// Per stage, per wave
+// Three launches per call, all on the caller's stream (the host never sees the lengths):
+//   1. paged_decode_plan_kernel (one workgroup): prefix sum of stage counts, run length, and for each
+//      column the sequence and stage it starts at.
+//   2. paged_decode_kernel: ncols x (hkv/HPW) workgroups of HPW waves; a workgroup takes HPW kv heads
+//      of its column's run (one head per wave), so it streams HPW*256 contiguous bytes per token.
+//      The first stage of the next piece (and its query rows) is already in flight while the last
+//      stage of the current piece is consumed: a wave never drains its load queue inside its run.
+//      A piece that covers a whole sequence is normalised and written to `out`; a piece that shares
+//      its sequence with other columns leaves (max, sum, unnormalised O) in one of the column's two
+//      partial slots (slot 0: the sequence began in an earlier column, slot 1: it began here).
+//   3. paged_decode_combine_kernel: merges the partials of sequences spread over several columns and
+//      writes zero rows for empty sequences.
+//
+// Inside a wave (one kv head, all hq/hkv query heads of its group served from one read of K and V)
+//   stage = 32 consecutive tokens (inside one cache block): 8 KiB of K + 8 KiB of V.  Stage i+1 is in
+//           flight from HBM into registers while stage i is consumed out of the wave's private LDS tile.
 //   S^T[token, qhead] = K[token, :] . Q^T            8 x v_mfma_f32_16x16x32_bf16 (K tile as A operand,
 //                                                     read back from LDS with a 16-byte XOR swizzle)
 //   online softmax over tokens (base-2 exponent, fp32 running max / sum per query head)
@@ -19,10 +30,8 @@
 //                                                     LDS through ds_read_b64_tr_b16 (transposing read)
 //   The accumulator layout of S^T is exactly the B-operand layout the second product needs, so P never
 //   moves between lanes.
-//
-// A sequence whose context fits one chunk is written straight to `out`; longer ones leave
-// (max, sum, unnormalised O) partials in the workspace for paged_decode_combine_kernel.
 #include "mops_common.h"
+#include <stdlib.h>
 
 namespace mops {
 
@@ -30,6 +39,9 @@ constexpr int kHeadDim = 128;
 constexpr int kStageTokens = 32;
 constexpr int kRowBytes = kHeadDim * 2;                  // one token, one kv head
 constexpr int kTileBytes = kStageTokens * kRowBytes;     // 8 KiB
+constexpr int kPlanThreads = 256;
+constexpr int kPlanLdsSeqs = 4096;                       // prefix array kept in LDS up to this batch
+constexpr int kHdrInts = 64;                             // workspace header: [0] total stages, [1] stages per column
 
 // Byte offset of 16-byte piece `slice` of token row `t` inside a swizzled LDS tile.
 __device__ __forceinline__ int tile_offset(int t, int slice) {
@@ -45,11 +57,14 @@ struct DecodeParams {
   const int32_t* block_table;
   int64_t block_table_row_stride;
   uint16_t* out;
-  float* ws_acc;   // [batch*hq, max_chunks, 128]
-  float* ws_ml;    // [batch*hq, max_chunks, 2]   (running max in the base-2 scaled domain, sum)
+  int32_t* hdr;        // [kHdrInts]
+  int32_t* prefix;     // [batch + 1] exclusive prefix sum of per-sequence stage counts
+  int32_t* col_start;  // [ncols][2]  first sequence of the column's run, stage offset inside it
+  float* ws_acc;       // [ncols][2][hq][128]
+  float* ws_ml;        // [ncols][2][hq][2]   (running max in the base-2 scaled domain, sum)
   int batch, hq, hkv, group;       // group = hq / hkv  (<= 16)
   int block_size, num_blocks, max_blocks_per_seq;
-  int chunk_tokens, max_chunks;
+  int ncols;
   float scale_log2;                // softmax_scale * log2(e)
 };
 
@@ -57,81 +72,203 @@ __device__ __forceinline__ int clamp_seqlen(int s, const DecodeParams& p) {
   const int cap = p.max_blocks_per_seq * p.block_size;
   return s < 0 ? 0 : (s > cap ? cap : s);
 }
+__device__ __forceinline__ int stages_of(int seqlen) { return (seqlen + kStageTokens - 1) / kStageTokens; }
 
-__global__ __launch_bounds__(kWave) void paged_decode_kernel(const DecodeParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kTileBytes];
-  unsigned char* const lds_k = lds;
-  unsigned char* const lds_v = lds + kTileBytes;
+// Scalar (constant-cache) load of a wave-uniform int that no kernel in flight writes.  Used inside
+// the main loop, where a vector load would have to wait behind the whole queue of KV loads.
+__device__ __forceinline__ int sload_i32(const int32_t* ptr) {
+  const uint64_t a = reinterpret_cast<uint64_t>(ptr);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  const uint64_t u = ((uint64_t)hi << 32) | lo;
+  int v;
+  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(u) : "memory");
+  return v;
+}
 
-  const int lane = threadIdx.x;
-  const int unit = blockIdx.x;
-  const int g = unit % p.hkv;
-  const int b = (unit / p.hkv) % p.batch;
-  const int c = unit / (p.hkv * p.batch);
+// ---------------------------------------------------------------------------------------------------
+// 1. plan
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kPlanThreads) void paged_decode_plan_kernel(const DecodeParams p) {
+  __shared__ int scan[kPlanThreads];
+  __shared__ int prefix_lds[kPlanLdsSeqs + 1];
+  const int tid = threadIdx.x;
+  const bool use_lds = p.batch <= kPlanLdsSeqs;
+  const int per_thread = (p.batch + kPlanThreads - 1) / kPlanThreads;
+  const int b0 = min(tid * per_thread, p.batch), b1 = min(b0 + per_thread, p.batch);
+  int mine = 0;
+  for (int b = b0; b < b1; ++b) mine += stages_of(clamp_seqlen(p.cache_seqlens[b], p));
+  scan[tid] = mine;
+  __syncthreads();
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    const int v = tid >= off ? scan[tid - off] : 0;
+    __syncthreads();
+    scan[tid] += v;
+    __syncthreads();
+  }
+  const int total = scan[kPlanThreads - 1];
+  int pos = scan[tid] - mine;
+  for (int b = b0; b < b1; ++b) {
+    p.prefix[b] = pos;
+    if (use_lds) prefix_lds[b] = pos;
+    pos += stages_of(clamp_seqlen(p.cache_seqlens[b], p));
+  }
+  if (tid == 0) {
+    p.prefix[p.batch] = total;
+    if (use_lds) prefix_lds[p.batch] = total;
+  }
+  const int per_col = max(1, (total + p.ncols - 1) / p.ncols);
+  if (tid == 0) {
+    p.hdr[0] = total;
+    p.hdr[1] = per_col;
+  }
+  __syncthreads();
+  const int* pre = use_lds ? prefix_lds : p.prefix;
+  for (int j = tid; j < p.ncols; j += kPlanThreads) {
+    const int64_t flat64 = (int64_t)j * per_col;
+    int b = 0, s = 0;
+    if (flat64 < total) {
+      const int flat = (int)flat64;
+      // largest b with prefix[b] <= flat; ties (empty sequences) resolve to the last of them,
+      // which is the non-empty one that owns the stage
+      int lo = 0, hi = p.batch;  // invariant: prefix[lo] <= flat < prefix[hi]
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (pre[mid] <= flat) lo = mid; else hi = mid;
+      }
+      b = lo;
+      s = flat - pre[lo];
+    }
+    p.col_start[2 * j] = b;
+    p.col_start[2 * j + 1] = s;
+  }
+}
 
-  const int seqlen = clamp_seqlen(p.cache_seqlens[b], p);
-  const int nchunks = (seqlen + p.chunk_tokens - 1) / p.chunk_tokens;
-  if (c >= (nchunks > 0 ? nchunks : 1)) return;
+// ---------------------------------------------------------------------------------------------------
+// 2. main kernel
+// ---------------------------------------------------------------------------------------------------
+struct Piece {       // wave-uniform: the part of one sequence that lies inside this column's run
+  int valid;
+  int b;
+  int tok_begin, tok_end, nstages;
+  int complete;      // covers the whole sequence: normalise and write `out` directly
+  int slot;          // partial slot of the column when not complete
+  int blk0;          // cache block of the first stage
+};
 
-  const int n = lane & 15;   // query head inside the group (MFMA column)
-  const int jj = lane >> 4;  // MFMA row quad / k slice
-  const int tok_begin = c * p.chunk_tokens;
-  const int tok_end = min(seqlen, tok_begin + p.chunk_tokens);
-  const int nstages = (tok_end - tok_begin + kStageTokens - 1) / kStageTokens;  // 0 when seqlen == 0
+template <int HPW>
+__global__ __launch_bounds__(kWave * HPW, 2) void paged_decode_kernel(const DecodeParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds_all[HPW * 2 * kTileBytes];
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  unsigned char* const lds_k = lds_all + wave * 2 * kTileBytes;
+  unsigned char* const lds_v = lds_k + kTileBytes;
 
+  const int n_hg = p.hkv / HPW;                      // head groups (workgroups) per column
+  const int col = blockIdx.x / n_hg;
+  const int g = (blockIdx.x % n_hg) * HPW + wave;    // this wave's kv head
+  const int total = p.hdr[0];
+  const int per_col = p.hdr[1];
+  const int64_t flat0 = (int64_t)col * per_col;
+  if (flat0 >= total) return;
+  int remaining = min(per_col, total - (int)flat0);  // stages left in this column's run
+
+  const int n = lane & 15;                           // query head inside the group (MFMA column)
+  const int jj = lane >> 4;                          // MFMA row quad / k slice
+  const int ld_tok = lane >> 4;                      // token (mod 4) this lane loads
+  const int ld_slice = lane & 15;                    // 16-byte piece of the 256-byte row
+  const int64_t tok_stride = (int64_t)p.hkv * kHeadDim;
+  const bool head_ok = n < p.group;
+
+  auto block_ok = [&](int blk) -> bool { return blk >= 0 && blk < p.num_blocks; };
+  auto table_at = [&](int b, int tok) -> int {
+    return sload_i32(p.block_table + (int64_t)b * p.block_table_row_stride + tok / p.block_size);
+  };
+  // piece of sequence b starting at its stage s, limited to `budget` stages
+  auto make_piece = [&](int b, int s, int budget) -> Piece {
+    Piece d;
+    const int seqlen = clamp_seqlen(sload_i32(p.cache_seqlens + b), p);
+    const int nst = stages_of(seqlen);
+    const int e = min(nst, s + budget);
+    d.valid = e > s;
+    d.b = b;
+    d.tok_begin = s * kStageTokens;
+    d.tok_end = min(seqlen, e * kStageTokens);
+    d.nstages = e - s;
+    d.complete = (s == 0 && e == nst);
+    d.slot = s > 0 ? 0 : 1;
+    d.blk0 = d.valid ? table_at(b, d.tok_begin) : -1;
+    return d;
+  };
+  // first non-empty sequence after b (the run still has stages left, so one exists)
+  auto next_piece = [&](int b, int budget) -> Piece {
+    Piece d;
+    d.valid = 0;
+    d.b = b;
+    d.tok_begin = d.tok_end = d.nstages = d.complete = d.slot = 0;
+    d.blk0 = -1;
+    if (budget <= 0) return d;
+    for (int nb = b + 1; nb < p.batch; ++nb) {
+      d = make_piece(nb, 0, budget);
+      if (d.valid) break;
+    }
+    return d;
+  };
+
+  // Per-lane byte offsets of the eight rows a lane loads per stage: fixed for the whole kernel, so an
+  // issue only has to form two wave-uniform base addresses.
+  uint32_t voff[8];
+#pragma unroll
+  for (int qi = 0; qi < 8; ++qi)
+    voff[qi] = (uint32_t)(((int64_t)(4 * qi + ld_tok) * tok_stride + (ld_slice << 3)) * 2);
+  u32x4 kreg[8], vreg[8];
+  auto issue_loads = [&](int tok0, int blk) {   // tok0: first token of the stage inside its sequence
+    const int64_t base = (((int64_t)blk * p.block_size + (tok0 % p.block_size)) * tok_stride + (int64_t)g * kHeadDim) * 2;
+    const char* kb = reinterpret_cast<const char*>(p.k_cache) + base;
+    const char* vb = reinterpret_cast<const char*>(p.v_cache) + base;
+#pragma unroll
+    for (int qi = 0; qi < 8; ++qi) {
+      kreg[qi] = load16_stream(kb + voff[qi]);
+      vreg[qi] = load16_stream(vb + voff[qi]);
+    }
+  };
   // Q as the B operand of S^T = K . Q^T: lane (n, jj) holds Q[g*group + n][(4*kb + jj)*8 .. +8).
-  bf16x8 qb[4];
-  {
-    const bool head_ok = n < p.group;
+  auto load_q = [&](int b, bf16x8 (&dst)[4]) {
     const uint16_t* qrow = p.q + (int64_t)b * p.q_batch_stride + (int64_t)(g * p.group + (head_ok ? n : 0)) * kHeadDim;
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
       u32x4 w = {0u, 0u, 0u, 0u};
       if (head_ok) w = load16(qrow + ((4 * kb + jj) << 3));
-      qb[kb] = __builtin_bit_cast(bf16x8, w);
-    }
-  }
-
-  const int32_t* table = p.block_table + (int64_t)b * p.block_table_row_stride;
-  const int64_t tok_stride = (int64_t)p.hkv * kHeadDim;  // elements between consecutive tokens of a block
-  const int ld_tok = lane >> 4;                           // token (mod 4) this lane loads
-  const int ld_slice = lane & 15;                         // 16-byte piece of the 256-byte row
-
-  u32x4 kreg[8], vreg[8];
-  auto issue_loads = [&](int stage, int blk) {
-    const int t0 = tok_begin + stage * kStageTokens;
-    const int64_t base = ((int64_t)blk * p.block_size + (t0 % p.block_size) + ld_tok) * tok_stride +
-                         (int64_t)g * kHeadDim + (ld_slice << 3);
-#pragma unroll
-    for (int qi = 0; qi < 8; ++qi) {
-      kreg[qi] = load16_stream(p.k_cache + base + (int64_t)(4 * qi) * tok_stride);
-      vreg[qi] = load16_stream(p.v_cache + base + (int64_t)(4 * qi) * tok_stride);
+      dst[kb] = __builtin_bit_cast(bf16x8, w);
     }
   };
-  auto block_of = [&](int stage) -> int {
-    const int t0 = tok_begin + stage * kStageTokens;
-    return table[t0 / p.block_size];
-  };
-  auto block_ok = [&](int blk) -> bool { return blk >= 0 && blk < p.num_blocks; };
 
+  Piece cur = make_piece(p.col_start[2 * col], p.col_start[2 * col + 1], remaining);
+  if (!cur.valid) return;  // cannot happen for a planned run
+
+  bf16x8 qb[4];
   f32x4 acc[8];
 #pragma unroll
   for (int dt = 0; dt < 8; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY;  // running max of scaled (base-2) scores for query head n
   float l_run = 0.f;        // this lane's share of the running sum
 
-  int blk_cur = nstages > 0 ? block_of(0) : -1;
-  int blk_next = nstages > 1 ? block_of(1) : -1;
-  if (nstages > 0 && block_ok(blk_cur)) issue_loads(0, blk_cur);
-  // Pin the wait for Q here, behind the first stage's loads, so the loop body never has to wait for
-  // "everything outstanding" on Q's account.
+  // Block of the stage whose data is in (or on its way to) the registers.  A table entry outside the
+  // cache is read as block 0 with every token masked, so control flow never depends on it.
+  int blk_ld = cur.blk0;
+  load_q(cur.b, qb);
+  issue_loads(cur.tok_begin, block_ok(blk_ld) ? blk_ld : 0);
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(qb[kb]));
 
-  for (int st = 0; st < nstages; ++st) {
-    const bool cur_ok = block_ok(blk_cur);
-    const int valid = min(kStageTokens, tok_end - (tok_begin + st * kStageTokens));
-    if (cur_ok) {
+  while (true) {
+    remaining -= cur.nstages;
+    // the piece after this one: looked up now, while this piece's first stage is still in flight
+    const Piece nxt = next_piece(cur.b, remaining);
+    int st = 0;
+    do {
+      const int tok0 = cur.tok_begin + st * kStageTokens;
+      const int valid = block_ok(blk_ld) ? min(kStageTokens, cur.tok_end - tok0) : 0;
       // registers -> LDS (swizzled); V rows past the end of the context become zeros so that a
       // zero probability times stale cache contents can never produce a NaN.
 #pragma unroll
@@ -148,13 +285,30 @@ __global__ __launch_bounds__(kWave) void paged_decode_kernel(const DecodeParams 
           if (t >= valid) *reinterpret_cast<u32x4*>(lds_v + tile_offset(t, ld_slice)) = u32x4{0u, 0u, 0u, 0u};
         }
       }
-    }
-    // next stage goes in flight before this one is consumed
-    const int blk_after = (st + 2 < nstages) ? block_of(st + 2) : -1;
-    if (st + 1 < nstages && block_ok(blk_next)) issue_loads(st + 1, blk_next);
-    __syncthreads();
+      // Everything older than the rows just consumed has landed; the only loads that can still be
+      // outstanding are a new piece's query rows.  Waiting for them here, with the queue empty, keeps
+      // the compute section free of a wait that would also cover the stage issued below.
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) asm volatile("" : "+v"(qb[kb]));
+      // ---- put the next stage in flight before this one is consumed: the next stage of this piece,
+      //      or the first stage (and the query rows) of the next piece
+      const bool last_stage = st + 1 >= cur.nstages;
+      {
+        int tok1 = tok0 + kStageTokens;
+        bool more = true;
+        if (!last_stage) {
+          if (tok1 % p.block_size == 0) blk_ld = table_at(cur.b, tok1);
+        } else {
+          tok1 = nxt.tok_begin;
+          blk_ld = nxt.blk0;
+          more = nxt.valid;
+        }
+        if (more) issue_loads(tok1, block_ok(blk_ld) ? blk_ld : 0);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-    if (cur_ok) {
       // ---- S^T = K . Q^T for the two 16-token tiles
       f32x4 s[2];
 #pragma unroll
@@ -217,59 +371,76 @@ __global__ __launch_bounds__(kWave) void paged_decode_kernel(const DecodeParams 
         const s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb, acc[dt], 0, 0, 0);
       }
-    }
-    __syncthreads();
-    blk_cur = blk_next;
-    blk_next = blk_after;
-  }
+      // the query rows are free now: on the last stage, fetch the next piece's into the same registers
+      if (last_stage && nxt.valid) load_q(nxt.b, qb);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      ++st;
+    } while (st < cur.nstages);
 
-  // total sum for query head n over the four row-quads
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
-
-  if (n >= p.group) return;
-  const int h = g * p.group + n;
-  if (nchunks <= 1) {
-    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    uint16_t* orow = p.out + ((int64_t)b * p.hq + h) * kHeadDim;
+    // ---- piece finished: total sum for query head n over the four row-quads, then write out
+    float l_tot = l_run + __shfl_xor(l_run, 16, kWave);
+    l_tot += __shfl_xor(l_tot, 32, kWave);
+    if (head_ok) {
+      const int h = g * p.group + n;
+      if (cur.complete) {
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        uint16_t* orow = p.out + ((int64_t)cur.b * p.hq + h) * kHeadDim;
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) {
-      u32x2 w;
-      w[0] = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
-      w[1] = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
-      *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * jj) = w;
-    }
-  } else {
-    const int64_t slot = ((int64_t)b * p.hq + h) * p.max_chunks + c;
-    float* arow = p.ws_acc + slot * kHeadDim;
+        for (int dt = 0; dt < 8; ++dt) {
+          u32x2 w;
+          w[0] = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
+          w[1] = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
+          *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * jj) = w;
+        }
+      } else {
+        const int64_t slot = ((int64_t)col * 2 + cur.slot) * p.hq + h;
+        float* arow = p.ws_acc + slot * kHeadDim;
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<f32x4*>(arow + 16 * dt + 4 * jj) = acc[dt];
-    if (jj == 0) {
-      p.ws_ml[2 * slot] = m_run;
-      p.ws_ml[2 * slot + 1] = l_run;
+        for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<f32x4*>(arow + 16 * dt + 4 * jj) = acc[dt];
+        if (jj == 0) {
+          p.ws_ml[2 * slot] = m_run;
+          p.ws_ml[2 * slot + 1] = l_tot;
+        }
+      }
     }
+    if (!nxt.valid) break;
+    cur = nxt;
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run = -INFINITY;
+    l_run = 0.f;
   }
 }
 
-// Merges the per-chunk partials of every (sequence, query head) that needed more than one chunk.
-// One wave per (b, h); lane owns two output elements.
+// ---------------------------------------------------------------------------------------------------
+// 3. combine: one wave per (sequence, query head); lane owns two output elements.
+// ---------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kWave) void paged_decode_combine_kernel(const DecodeParams p) {
   const int bh = blockIdx.x;
   const int b = bh / p.hq;
-  const int seqlen = clamp_seqlen(p.cache_seqlens[b], p);
-  const int nchunks = (seqlen + p.chunk_tokens - 1) / p.chunk_tokens;
-  if (nchunks <= 1) return;
+  const int h = bh % p.hq;
   const int lane = threadIdx.x;
-  const float* ml = p.ws_ml + (int64_t)bh * p.max_chunks * 2;
-  const float* accp = p.ws_acc + (int64_t)bh * p.max_chunks * kHeadDim + 2 * lane;
+  const int f0 = p.prefix[b], f1 = p.prefix[b + 1];
+  if (f1 == f0) {  // an empty context attends to nothing: zeros
+    reinterpret_cast<uint32_t*>(p.out + (int64_t)bh * kHeadDim)[lane] = 0u;
+    return;
+  }
+  const int per_col = p.hdr[1];
+  const int j0 = f0 / per_col, j1 = (f1 - 1) / per_col;
+  if (j0 == j1) return;  // one piece: written directly by the main kernel
+  // partial of column j: slot 1 in the column where the sequence begins, slot 0 in the following ones
+  auto slot_of = [&](int j) -> int64_t { return ((int64_t)j * 2 + (j == j0 ? 1 : 0)) * p.hq + h; };
   float m = -INFINITY;
-  for (int c = 0; c < nchunks; ++c) m = fmaxf(m, ml[2 * c]);
+  for (int j = j0; j <= j1; ++j) m = fmaxf(m, p.ws_ml[2 * slot_of(j)]);
   const float m_safe = (m == -INFINITY) ? 0.f : m;
   float l = 0.f, o0 = 0.f, o1 = 0.f;
-  for (int c = 0; c < nchunks; ++c) {
-    const float w = __builtin_amdgcn_exp2f(ml[2 * c] - m_safe);
-    l += w * ml[2 * c + 1];
-    const float2 a = *reinterpret_cast<const float2*>(accp + (int64_t)c * kHeadDim);
+  for (int j = j0; j <= j1; ++j) {
+    const int64_t sl = slot_of(j);
+    const float w = __builtin_amdgcn_exp2f(p.ws_ml[2 * sl] - m_safe);
+    l += w * p.ws_ml[2 * sl + 1];
+    const float2 a = *reinterpret_cast<const float2*>(p.ws_acc + sl * kHeadDim + 2 * lane);
     o0 += w * a.x;
     o1 += w * a.y;
   }
@@ -277,19 +448,58 @@ __global__ __launch_bounds__(kWave) void paged_decode_combine_kernel(const Decod
   reinterpret_cast<uint32_t*>(p.out + (int64_t)bh * kHeadDim)[lane] = pack_bf16x2(o0 * inv, o1 * inv);
 }
 
-// Chunk length (tokens, multiple of the stage) chosen from launch-time upper bounds only: enough
-// units to keep every SIMD of the 256 CUs busy for several rounds, but not so many that the
-// partials traffic shows up next to the KV stream.
-static int choose_chunk_tokens(int64_t batch, int64_t hkv, int64_t max_tokens) {
-  const int64_t target_units = 16384;
-  int64_t chunk = (batch * hkv * max_tokens + target_units - 1) / target_units;
-  chunk = (chunk + kStageTokens - 1) / kStageTokens * kStageTokens;
-  if (chunk < 2 * kStageTokens) chunk = 2 * kStageTokens;
-  if (chunk > 512) chunk = 512;
-  return (int)chunk;
+// ---------------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------------
+static int env_int(const char* name) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : 0;
+}
+
+// Waves (= kv heads) per workgroup: 2 streams 512 contiguous bytes per token per workgroup and still
+// leaves four independent workgroups per CU.
+static int choose_hpw(int hkv) {
+  static const int forced = env_int("MOPS_HIP_DECODE_HPW");  // tuning override: 1, 2, 4 or 8
+  int want = (forced == 1 || forced == 2 || forced == 4 || forced == 8) ? forced : 2;
+  while (want > 1 && hkv % want != 0) want >>= 1;
+  return want;
+}
+
+static int device_cu_count() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    return n;
+  }();
+  return cus;
+}
+
+// Columns of the flat split: every CU holds 8 waves (16 KiB of LDS tiles each, two per SIMD), a
+// column needs hkv waves.
+static int choose_ncols(int64_t hkv) {
+  static const int forced = env_int("MOPS_HIP_DECODE_NCOLS");  // tuning override
+  if (forced > 0) return forced;
+  const int64_t n = (int64_t)device_cu_count() * 8 / hkv;
+  return (int)(n < 1 ? 1 : n);
 }
 
 static int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+struct WorkspaceLayout {
+  int64_t hdr, prefix, col_start, acc, ml, total;
+};
+
+static WorkspaceLayout workspace_layout(int64_t batch, int64_t hq, int64_t ncols) {
+  WorkspaceLayout w;
+  w.hdr = 0;
+  w.prefix = align_up(kHdrInts * 4, 256);
+  w.col_start = w.prefix + align_up((batch + 1) * 4, 256);
+  w.acc = w.col_start + align_up(ncols * 2 * 4, 256);
+  w.ml = w.acc + align_up(ncols * 2 * hq * kHeadDim * 4, 256);
+  w.total = w.ml + align_up(ncols * 2 * hq * 2 * 4, 256);
+  return w;
+}
 
 }  // namespace mops
 
@@ -297,11 +507,7 @@ extern "C" int64_t mops_hip_paged_decode_workspace_bytes(int64_t batch, int64_t 
                                                          int64_t max_blocks_per_seq, int64_t block_size) {
   using namespace mops;
   if (batch <= 0 || hq <= 0 || hkv <= 0 || max_blocks_per_seq <= 0 || block_size <= 0) return 0;
-  const int64_t max_tokens = max_blocks_per_seq * block_size;
-  const int chunk = choose_chunk_tokens(batch, hkv, max_tokens);
-  const int64_t max_chunks = (max_tokens + chunk - 1) / chunk;
-  if (max_chunks <= 1) return 256;
-  return align_up(batch * hq * max_chunks * kHeadDim * 4, 256) + align_up(batch * hq * max_chunks * 2 * 4, 256);
+  return workspace_layout(batch, hq, choose_ncols(hkv)).total;
 }
 
 extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
@@ -319,18 +525,15 @@ extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_st
     return MOPS_HIP_EINVAL;
   if (batch == 0) return MOPS_HIP_OK;
   if (!q || !k_cache || !v_cache || !cache_seqlens || !block_table || !out) return MOPS_HIP_EINVAL;
-  if (hq % hkv != 0 || block_table_row_stride < max_blocks_per_seq) return MOPS_HIP_EINVAL;
+  if (hq % hkv != 0 || block_table_row_stride < max_blocks_per_seq || num_blocks == 0) return MOPS_HIP_EINVAL;
   if (q_batch_stride < hq * head_dim) return MOPS_HIP_EINVAL;
   if (head_dim != kHeadDim || hq / hkv > 16 || block_size % kStageTokens != 0) return MOPS_HIP_EUNSUPPORTED;
-  if (batch > (1 << 20) || hq > 4096 || max_blocks_per_seq * block_size > (1 << 24) ||
+  if (batch >= (1 << 20) || hq > 4096 || hkv > 1024 || max_blocks_per_seq * block_size > (1 << 24) ||
       num_blocks * block_size > (int64_t)0x7fffffff)
     return MOPS_HIP_EUNSUPPORTED;
   if ((q_batch_stride & 7)) return MOPS_HIP_EALIGN;
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out)) return MOPS_HIP_EALIGN;
-  if (max_blocks_per_seq == 0) {
-    hipError_t e = hipMemsetAsync(out, 0, (size_t)(batch * hq * kHeadDim * 2), (hipStream_t)stream);
-    return e == hipSuccess ? MOPS_HIP_OK : MOPS_HIP_ELAUNCH;
-  }
+  hipStream_t s = (hipStream_t)stream;
 
   DecodeParams p;
   p.q = (const uint16_t*)q;
@@ -348,28 +551,32 @@ extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_st
   p.block_size = (int)block_size;
   p.num_blocks = (int)num_blocks;
   p.max_blocks_per_seq = (int)max_blocks_per_seq;
-  const int64_t max_tokens = max_blocks_per_seq * block_size;
-  p.chunk_tokens = choose_chunk_tokens(batch, hkv, max_tokens);
-  p.max_chunks = (int)((max_tokens + p.chunk_tokens - 1) / p.chunk_tokens);
+  p.ncols = choose_ncols(hkv);
   p.scale_log2 = softmax_scale * 1.44269504088896340736f;
-  p.ws_acc = nullptr;
-  p.ws_ml = nullptr;
-  if (p.max_chunks > 1) {
-    const int64_t need = mops_hip_paged_decode_workspace_bytes(batch, hq, hkv, max_blocks_per_seq, block_size);
-    if (!workspace || workspace_bytes < need) return MOPS_HIP_EWORKSPACE;
-    if (reinterpret_cast<uintptr_t>(workspace) & 255u) return MOPS_HIP_EALIGN;
-    p.ws_acc = (float*)workspace;
-    p.ws_ml = (float*)((char*)workspace + align_up(batch * hq * p.max_chunks * kHeadDim * 4, 256));
-  }
-  const int64_t units = batch * hkv * p.max_chunks;
-  if (units > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
-  hipLaunchKernelGGL(paged_decode_kernel, dim3((unsigned)units), dim3(kWave), 0, (hipStream_t)stream, p);
+  const WorkspaceLayout w = workspace_layout(batch, hq, p.ncols);
+  if (!workspace || workspace_bytes < w.total) return MOPS_HIP_EWORKSPACE;
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return MOPS_HIP_EALIGN;
+  char* base = (char*)workspace;
+  p.hdr = (int32_t*)(base + w.hdr);
+  p.prefix = (int32_t*)(base + w.prefix);
+  p.col_start = (int32_t*)(base + w.col_start);
+  p.ws_acc = (float*)(base + w.acc);
+  p.ws_ml = (float*)(base + w.ml);
+
+  hipLaunchKernelGGL(paged_decode_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, p);
   int st = finish_launch();
   if (st != MOPS_HIP_OK) return st;
-  if (p.max_chunks > 1) {
-    hipLaunchKernelGGL(paged_decode_combine_kernel, dim3((unsigned)(batch * hq)), dim3(kWave), 0,
-                       (hipStream_t)stream, p);
-    st = finish_launch();
+
+  const int hpw = choose_hpw(p.hkv);
+  const dim3 grid((unsigned)((int64_t)p.ncols * (p.hkv / hpw))), block((unsigned)(kWave * hpw));
+  switch (hpw) {
+    case 8: hipLaunchKernelGGL(paged_decode_kernel<8>, grid, block, 0, s, p); break;
+    case 4: hipLaunchKernelGGL(paged_decode_kernel<4>, grid, block, 0, s, p); break;
+    case 2: hipLaunchKernelGGL(paged_decode_kernel<2>, grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL(paged_decode_kernel<1>, grid, block, 0, s, p); break;
   }
-  return st;
+  st = finish_launch();
+  if (st != MOPS_HIP_OK) return st;
+  hipLaunchKernelGGL(paged_decode_combine_kernel, dim3((unsigned)(batch * hq)), dim3(kWave), 0, s, p);
+  return finish_launch();
 }
