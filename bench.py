@@ -6,6 +6,8 @@ query token each, 16 q heads / 8 kv heads, head_dim 128, context uniform in [512
 A step is one flash_attn_with_kvcache call over the whole batch, KV cache resident in HBM.
 `--op` selects another operator of the hot path (same JSON format, its own metric):
   decode (default) | decode8b | prefill | store | add_rms | rms | embedding
+  copy = a plain 1 GiB device-to-device tensor copy (not a mops op): the known-size kernel against which
+         the FETCH_SIZE / WRITE_SIZE counters of a profile are calibrated.
 
 Prints ONE JSON line on stdout.  `roofline` is computed from HIP-event time of the op on its launch
 stream; `cpu_baseline` times the CPU restatement of the reference's torch backend (oracle/) on a
@@ -29,7 +31,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding"])
+                    choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
@@ -110,7 +112,7 @@ def main():
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401
             ref = mops.get_op("flash_attn_with_kvcache", "torch")
-            n = 32
+            n = 64
             sub_tbl = table[:n]
             used = sub_tbl[sub_tbl >= 0].long()
             remap = torch.full((nblk,), -1, dtype=torch.int32)
@@ -121,12 +123,13 @@ def main():
             qc = q[:n].cpu()
             lens = torch.tensor(ctx[:n], dtype=torch.int32)
             ref(qc, kc, vc, cache_seqlens=lens, block_table=tbl, softmax_scale=scale)
-            ts = []
-            for _ in range(3):
+            ts, t_start = [], time.perf_counter()
+            while len(ts) < 5 or (time.perf_counter() - t_start < 12.0 and len(ts) < 400):
                 t0 = time.perf_counter()
                 ref(qc, kc, vc, cache_seqlens=lens, block_table=tbl, softmax_scale=scale)
                 ts.append(time.perf_counter() - t0)
-            return sorted(ts)[1], f"first {n} of {bsz} sequences, median of 3", W.decode_bytes(ctx[:n], hq, hkv, max_blocks)
+            return (sorted(ts)[len(ts) // 2], f"first {n} of {bsz} sequences, median of {len(ts)} passes (~12 s of CPU work)",
+                    W.decode_bytes(ctx[:n], hq, hkv, max_blocks))
 
     elif args.op == "prefill":
         lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
@@ -223,6 +226,20 @@ def main():
                 ref(*a)
                 ts.append(time.perf_counter() - t0)
             return sorted(ts)[3], "whole batch, median of 7", work
+
+    elif args.op == "copy":
+        nbytes = 1 << 30
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+
+        def step(i):
+            return dst.copy_(src)
+
+        work = float(2 * nbytes)
+        metric, unit = "device_copy_GBps", "GB/s"
+        config = {"workload": "calibration: 1 GiB device-to-device copy (reads 1 GiB, writes 1 GiB)", "bytes": nbytes}
+        kernel_name = "torch elementwise copy"
+        cpu_fn = None
 
     else:  # embedding
         vocab, hidden, n_ids = 151936, 4096, 512

@@ -24,8 +24,12 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   __bf16 b = (__bf16)f;
   return (uint32_t)__builtin_bit_cast(unsigned short, b);
 }
+// Two fp32 -> one dword of two bf16 (lo in bits 0..15), one v_cvt_pk_bf16_f32.
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 __device__ __forceinline__ float round_to_bf16(float f) { return (float)(__bf16)f; }
 

@@ -27,8 +27,13 @@ constexpr int kPThreads = 256;
 constexpr int kPRowBytes = kPD * 2;
 constexpr int kPTileBytes = kPBN * kPRowBytes;  // 16 KiB
 
+// Byte offset of 16-byte piece `slice` of token row `t` inside an LDS tile.  The piece index is XORed
+// with the row's low four bits with the bit pairs swapped: 16 consecutive rows at one slice (the K
+// operand read) and 4 consecutive rows x 4 consecutive slices (the transposing V read) both spread
+// over all 64 banks.
 __device__ __forceinline__ int ptile_offset(int t, int slice) {
-  return t * kPRowBytes + ((slice ^ (t & 15)) << 4);
+  const int g = ((t & 3) << 2) | ((t >> 2) & 3);
+  return t * kPRowBytes + ((slice ^ g) << 4);
 }
 
 struct PrefillParams {
@@ -142,33 +147,36 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
           s[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), qb[kb], s[tt], 0, 0, 0);
         }
       }
-      // ---- scale, causal mask (only where the tile crosses the diagonal), running max
+      // ---- causal mask (only where the tile crosses the diagonal), running max of the raw scores;
+      //      the softmax scale is folded into the exponent: p = 2^(s*c - m*c)
       const bool need_mask = j0 + kPBN - 1 > wave_row0;
       float m_loc = -INFINITY;
+      if (need_mask) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
+            s[tt][r] = key <= my_row ? s[tt][r] : -INFINITY;
+          }
+      }
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float x = s[tt][r] * p.scale_log2;
-          if (need_mask) {
-            const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
-            x = key <= my_row ? x : -INFINITY;
-          }
-          s[tt][r] = x;
-          m_loc = fmaxf(m_loc, x);
-        }
+        for (int r = 0; r < 16; ++r) m_loc = fmaxf(m_loc, s[tt][r]);
       m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, kWave));
-      const float m_new = fmaxf(m_run, m_loc);
+      const float m_new = fmaxf(m_run, m_loc);                  // raw-score domain
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+      const float mc = m_safe * p.scale_log2;
+      const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - mc);
       float psum = 0.f;
       u32x4 pw[4];  // P^T as B operand for the four 16-token k blocks
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(s[tt][r] - m_safe);
-          const float p1 = __builtin_amdgcn_exp2f(s[tt][r + 1] - m_safe);
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r], p.scale_log2, -mc));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc));
           psum += p0 + p1;
           pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(p0, p1);
         }
