@@ -70,6 +70,7 @@ def main():
         return out
 
     cpu_fn = None      # () -> (seconds, description, units_done)  on a bounded sample
+    measured_traffic = None
     bound = "hbm"
     dtype = "bf16"
 
@@ -107,7 +108,10 @@ def main():
         config = {"workload": name, "batch": bsz, "q_heads": hq, "kv_heads": hkv, "head_dim": W.HEAD_DIM,
                   "block_size": W.BLOCK_SIZE, "context": f"uniform[{lo},{hi}] seed {args.seed}",
                   "context_tokens": sum(ctx), "kv_buffers_rotated": n_copies}
-        kernel_name = "paged_decode_kernel (+ paged_decode_combine_kernel)"
+        kernel_name = "paged_decode_kernel (+ paged_decode_plan_kernel, paged_decode_combine_kernel)"
+        # HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this exact
+        # workload (profiles/hbm_traffic_decode_prefill.txt); only valid for the default seed
+        measured_traffic = 2497.6e6 if (args.op == "decode" and args.seed == 0) else None
 
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401
@@ -296,7 +300,7 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic", "config": config,
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": runit,
-                     "frac": round(achieved / peak, 4), "traffic": None, "kernel": kernel_name,
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic, "kernel": kernel_name,
                      "algorithmic_work_per_launch": work, "event_ms_per_launch": round(ev_ms, 5),
                      "event_ms_min": round(min(per_step_ms), 5)},
     }
