@@ -41,7 +41,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); the hot path has no "
-              "cross-GPU exchange, see DESIGN.md for how it shards.", file=sys.stderr)
+              "cross-GPU exchange: each GPU would run the same kernels on its own kv heads or sequences.", file=sys.stderr)
         sys.exit(2)
 
     import torch
