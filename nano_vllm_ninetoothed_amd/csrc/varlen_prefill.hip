@@ -3,20 +3,27 @@
 //
 // Work decomposition
 //   workgroup (256 lanes, 4 waves) = one 128-row Q tile of one sequence for one query head; wave w owns
-//   rows 32w..32w+31.  Workgroups are numbered so that the query heads of one kv group are neighbours
-//   (their K/V tiles hit in L2) and the tiles with the longest causal prefix are dispatched first.
-//   The launch is sized from max_seqlen; tiles past a sequence's end exit at once.
+//   rows 32w..32w+31.  The launch is sized from max_seqlen (tiles past a sequence's end exit at once),
+//   the tiles with the longest causal prefix are dispatched first, and with 8 kv heads the workgroup id
+//   is decoded so that id % 8 — the XCD a workgroup lands on — is the kv head: each XCD's L2 then only
+//   ever holds one kv head's K/V.
 //
-// Per 64-token K/V tile (double-buffered in LDS, next tile in flight from HBM into registers)
-//   S^T[token, qrow] = K . Q^T        16 x v_mfma_f32_32x32x16_bf16 per wave; Q^T lives in registers as
-//                                      the B operand for the whole kernel, K rows are read from LDS
-//                                      with a 16-byte XOR swizzle
-//   online softmax down the token axis: each lane owns one q row, so max/sum are register-local
-//                                      plus one cross-half exchange
-//   O^T[d, qrow]   += V^T . P^T        16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
+// Per 64-token K/V tile (double-buffered in LDS, one workgroup barrier per tile, next tile in flight from
+// HBM into registers)
+//   S^T = K . Q^T                      16 x v_mfma_f32_32x32x16_bf16 per wave; Q^T stays in registers as
+//                                      the B operand; the K operand reads run four MFMAs ahead of use
+//   softmax down the token axis:       each lane owns one q row, so max/sum are register-local plus one
+//                                      half-wave swap (v_permlane32_swap); the scale is folded into the
+//                                      exponent, the causal mask is applied on a wave's last tile only
+//   O^T += V^T . P^T                   16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
 //                                      already the B-operand layout, V^T comes out of LDS through
-//                                      ds_read_b64_tr_b16
+//                                      ds_read_b64_tr_b16, also issued ahead of the MFMAs that use it
+//
+// LDS rows are padded instead of swizzled (K rows 272 B apart, V rows 320 B apart): the K operand read
+// (16 consecutive rows, one 16-byte piece) and the transposing V read (4 rows x 4 pieces) each cover
+// all 64 banks once, and every address a lane needs is one base register plus an immediate.
 #include "mops_common.h"
+#include <type_traits>
 
 namespace mops {
 
@@ -24,17 +31,10 @@ constexpr int kPD = 128;            // head dim
 constexpr int kPBM = 128;           // q rows per workgroup
 constexpr int kPBN = 64;            // kv tokens per tile
 constexpr int kPThreads = 256;
-constexpr int kPRowBytes = kPD * 2;
-constexpr int kPTileBytes = kPBN * kPRowBytes;  // 16 KiB
-
-// Byte offset of 16-byte piece `slice` of token row `t` inside an LDS tile.  The piece index is XORed
-// with the row's low four bits with the bit pairs swapped: 16 consecutive rows at one slice (the K
-// operand read) and 4 consecutive rows x 4 consecutive slices (the transposing V read) both spread
-// over all 64 banks.
-__device__ __forceinline__ int ptile_offset(int t, int slice) {
-  const int g = ((t & 3) << 2) | ((t >> 2) & 3);
-  return t * kPRowBytes + ((slice ^ g) << 4);
-}
+constexpr int kPKStride = 272;      // bytes between K rows in LDS
+constexpr int kPVStride = 320;      // bytes between V rows in LDS
+constexpr int kPKTile = kPBN * kPKStride;   // 17408
+constexpr int kPVTile = kPBN * kPVStride;   // 20480
 
 struct PrefillParams {
   const uint16_t* q;
@@ -47,13 +47,35 @@ struct PrefillParams {
   float scale_log2;
 };
 
-__global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[4 * kPTileBytes];  // [buf][K|V]
+// max / sum across the two 32-lane halves of the wave; every lane gets the result
+__device__ __forceinline__ float half_swap_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
+__global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPKTile + 2 * kPVTile];  // K[2] then V[2]
+  unsigned char* const lds_k = lds;
+  unsigned char* const lds_v = lds + 2 * kPKTile;
+
+  // ---- workgroup id -> (q tile m, sequence b, query head h)
   const int idx = blockIdx.x;
-  const int h = idx % p.hq;
-  const int b = (idx / p.hq) % p.batch;
-  const int m = p.m_tiles - 1 - idx / (p.hq * p.batch);
+  int h, rest;
+  if (p.hkv == 8) {  // id % 8 is the XCD: make it the kv head
+    const int g8 = idx & 7;
+    const int r = (idx >> 3) % p.group;
+    rest = (idx >> 3) / p.group;
+    h = g8 * p.group + r;
+  } else {
+    h = idx % p.hq;
+    rest = idx / p.hq;
+  }
+  const int b = rest % p.batch;
+  const int m = p.m_tiles - 1 - rest / p.batch;
   const int seq_begin = p.cu_seqlens[b];
   const int seq_len = min(p.cu_seqlens[b + 1], p.total_tokens) - seq_begin;
   const int q0 = m * kPBM;
@@ -70,6 +92,9 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   const int ntiles = (kv_end + kPBN - 1) / kPBN;
   const int wave_row0 = q0 + 32 * wave;          // first q row (sequence-relative) of this wave
   const int my_row = wave_row0 + n;
+  // tiles this wave has to look at: those holding a key visible to one of its rows.  Only the last of
+  // them crosses the diagonal (or the end of the sequence) and needs the mask.
+  const int my_tiles = min(ntiles, (wave_row0 + 31) / kPBN + 1);
 
   // ---- Q^T as B operand: lane (n, jj) holds Q[my_row][16*kb + 8*jj .. +8) for kb = 0..7
   bf16x8 qb[8];
@@ -87,31 +112,57 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   // ---- cooperative tile loads: thread moves 16-byte piece (tid & 15) of rows (tid >> 4) + 16*i
   const int ld_row = tid >> 4;
   const int ld_slice = tid & 15;
-  const uint16_t* kbase = p.k + (int64_t)seq_begin * p.k_ts + (int64_t)g * kPD + (ld_slice << 3);
-  const uint16_t* vbase = p.v + (int64_t)seq_begin * p.v_ts + (int64_t)g * kPD + (ld_slice << 3);
-  u32x4 kreg[4], vreg[4];
-  auto issue_loads = [&](int tile) {
+  const uint16_t* kptr = p.k + (int64_t)(seq_begin + ld_row) * p.k_ts + (int64_t)g * kPD + (ld_slice << 3);
+  const uint16_t* vptr = p.v + (int64_t)(seq_begin + ld_row) * p.v_ts + (int64_t)g * kPD + (ld_slice << 3);
+  auto load_tile = [&](const uint16_t* base, int64_t ts, int tile, u32x4 (&r)[4]) {
+    const uint16_t* src = base + (int64_t)tile * kPBN * ts;
+    if ((tile + 1) * kPBN <= seq_len) {  // whole tile inside the sequence
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int t = tile * kPBN + ld_row + 16 * i;
-      u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-      if (t < seq_len) {
-        kk = load16(kbase + (int64_t)t * p.k_ts);
-        vv = load16(vbase + (int64_t)t * p.v_ts);
+      for (int i = 0; i < 4; ++i) r[i] = load16(src + (int64_t)(16 * i) * ts);
+    } else {                             // rows past the sequence read as zeros
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = tile * kPBN + ld_row + 16 * i;
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (t < seq_len) x = load16(src + (int64_t)(16 * i) * ts);
+        r[i] = x;
       }
-      kreg[i] = kk;
-      vreg[i] = vv;
     }
   };
-  auto store_tile = [&](int buf) {
-    unsigned char* kt = lds + buf * 2 * kPTileBytes;
-    unsigned char* vt = kt + kPTileBytes;
+  const int st_k = ld_row * kPKStride + (ld_slice << 4);
+  const int st_v = ld_row * kPVStride + (ld_slice << 4);
+  auto store_k = [&](int buf, const u32x4 (&r)[4]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int off = ptile_offset(ld_row + 16 * i, ld_slice);
-      *reinterpret_cast<u32x4*>(kt + off) = kreg[i];
-      *reinterpret_cast<u32x4*>(vt + off) = vreg[i];
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds_k + buf * kPKTile + st_k + 16 * i * kPKStride) = r[i];
+  };
+  auto store_v = [&](int buf, const u32x4 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds_v + buf * kPVTile + st_v + 16 * i * kPVStride) = r[i];
+  };
+  // S^T = K . Q^T for one 64-token tile resident in LDS; lane (n, jj) reads row 32*tt + n, piece 2*kb + jj
+  const int rd_k = n * kPKStride + (jj << 4);
+  auto qk_tile = [&](int buf, f32x16 (&s)[2]) {
+    const unsigned char* kt = lds_k + buf * kPKTile + rd_k;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 8; ++kb)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(kt + tt * 32 * kPKStride + kb * 32);
+        s[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), qb[kb], s[tt], 0, 0, 0);
+      }
+    // issue order: four operand reads up front, then one read per MFMA, so LDS latency hides behind
+    // the matrix pipe instead of in front of every MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
   };
 
   f32x16 acc[4];
@@ -119,101 +170,99 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = -INFINITY;  // running max of the raw scores of row my_row
+  float l_run = 0.f;        // this lane's share of the running sum
 
-  issue_loads(0);
+  // transposing V read: 16-lane group (d half, jj); lane addresses token row src_row of a 4-row set and
+  // the 4-wide d chunk src_chunk of the group's 16-wide window
+  const int rd_v = (4 * jj + ((lane & 15) >> 2)) * kPVStride + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3);
+
+  // online softmax of one tile's scores (already in s) and O^T += V^T . P^T
+  auto softmax_pv = [&](f32x16 (&s)[2], int buf, int j0, auto masked) {
+    if (decltype(masked)::value) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
+          s[tt][r] = key <= my_row ? s[tt][r] : -INFINITY;
+        }
+    }
+    float m_loc = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+    for (int r = 1; r < 16; ++r) m_loc = fmaxf(m_loc, fmaxf(s[0][r], s[1][r]));
+    m_loc = half_swap_max(m_loc);
+    const float m_new = fmaxf(m_run, m_loc);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float mc = m_safe * p.scale_log2;
+    const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - mc);
+    float psum = 0.f;
+    u32x4 pw[4];  // P^T as B operand for the four 16-token k blocks
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r], p.scale_log2, -mc));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc));
+        psum += p0 + p1;
+        pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(p0, p1);
+      }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
+    }
+    const unsigned char* vt = lds_v + buf * kPVTile + rd_v;
+#pragma unroll
+    for (int kb2 = 0; kb2 < 4; ++kb2) {
+      const bf16x8 pb = __builtin_bit_cast(bf16x8, pw[kb2]);
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        // token rows 16*kb2 + 4*jj + src_row (+8 for the upper four), d = 32*dt + 16*half + 4*chunk ..
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)(vt + 16 * kb2 * kPVStride + 64 * dt));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)(vt + (16 * kb2 + 8) * kPVStride + 64 * dt));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), pb, acc[dt], 0, 0, 0);
+      }
+    }
+    // issue order: the transposing reads of four MFMAs up front, then two reads per MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+  };
+
+  // ---- tile loop: tile i+1 is in flight into registers while tile i is consumed out of LDS
+  u32x4 kreg[4], vreg[4];
+  load_tile(kptr, p.k_ts, 0, kreg);
+  load_tile(vptr, p.v_ts, 0, vreg);
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
-
+  f32x16 s[2];
   for (int tile = 0; tile < ntiles; ++tile) {
     const int buf = tile & 1;
-    store_tile(buf);
-    __syncthreads();
-    if (tile + 1 < ntiles) issue_loads(tile + 1);
-
-    const int j0 = tile * kPBN;
-    if (j0 <= wave_row0 + 31) {  // some key of the tile is visible to some row of this wave
-      const unsigned char* kt = lds + buf * 2 * kPTileBytes;
-      const unsigned char* vt = kt + kPTileBytes;
-      // ---- S^T = K . Q^T : two 32-token row tiles
-      f32x16 s[2];
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 8; ++kb) {
-          const u32x4 w = *reinterpret_cast<const u32x4*>(kt + ptile_offset(32 * tt + n, 2 * kb + jj));
-          s[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), qb[kb], s[tt], 0, 0, 0);
-        }
-      }
-      // ---- causal mask (only where the tile crosses the diagonal), running max of the raw scores;
-      //      the softmax scale is folded into the exponent: p = 2^(s*c - m*c)
-      const bool need_mask = j0 + kPBN - 1 > wave_row0;
-      float m_loc = -INFINITY;
-      if (need_mask) {
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
-            s[tt][r] = key <= my_row ? s[tt][r] : -INFINITY;
-          }
-      }
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) m_loc = fmaxf(m_loc, s[tt][r]);
-      m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, kWave));
-      const float m_new = fmaxf(m_run, m_loc);                  // raw-score domain
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float mc = m_safe * p.scale_log2;
-      const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - mc);
-      float psum = 0.f;
-      u32x4 pw[4];  // P^T as B operand for the four 16-token k blocks
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r], p.scale_log2, -mc));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc));
-          psum += p0 + p1;
-          pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(p0, p1);
-        }
-      l_run = l_run * alpha + psum;
-      m_run = m_new;
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
-      }
-      // ---- O^T += V^T . P^T
-      const int grp = lane >> 4;              // 16-lane group: (d half, jj)
-      const int src_row = (lane & 15) >> 2;   // token row this lane addresses inside a 4-row set
-      const int src_chunk = lane & 3;         // 4-wide d chunk inside the 16-wide window
-      const int d_half = grp & 1;
-#pragma unroll
-      for (int kb2 = 0; kb2 < 4; ++kb2) {
-        const bf16x8 pb = __builtin_bit_cast(bf16x8, pw[kb2]);
-        const int t_lo = 16 * kb2 + 4 * jj + src_row;
-        const int t_hi = t_lo + 8;
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          const int d0 = 32 * dt + 16 * d_half + 4 * src_chunk;  // first of 4 consecutive d
-          const int slice = d0 >> 3;
-          const int sub = (d0 & 7) << 1;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(vt + ptile_offset(t_lo, slice) + sub));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(vt + ptile_offset(t_hi, slice) + sub));
-          typedef short s16x8 __attribute__((ext_vector_type(8)));
-          const s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), pb, acc[dt], 0, 0, 0);
-        }
-      }
+    store_k(buf, kreg);
+    store_v(buf, vreg);
+    __syncthreads();   // tile visible to all waves; the other buffer (tile-1) is free once everyone is here
+    if (tile + 1 < ntiles) {
+      load_tile(kptr, p.k_ts, tile + 1, kreg);
+      load_tile(vptr, p.v_ts, tile + 1, vreg);
+    }
+    if (tile < my_tiles) {
+      qk_tile(buf, s);
+      if (tile + 1 == my_tiles) softmax_pv(s, buf, tile * kPBN, std::true_type{});
+      else softmax_pv(s, buf, tile * kPBN, std::false_type{});
     }
   }
 
-  l_run += __shfl_xor(l_run, 32, kWave);
+  l_run = half_swap_sum(l_run);
   if (my_row < seq_len) {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     uint16_t* orow = p.out + (int64_t)(seq_begin + my_row) * p.o_ts + (int64_t)h * kPD;
