@@ -6,6 +6,9 @@ query token each, 16 q heads / 8 kv heads, head_dim 128, context uniform in [512
 A step is one flash_attn_with_kvcache call over the whole batch, KV cache resident in HBM.
 `--op` selects another operator of the hot path (same JSON format, its own metric):
   decode (default) | decode8b | prefill | store | add_rms | rms | embedding
+  e2e  = end-to-end generation on a randomly initialised Qwen3-0.6B-shaped model through the engine
+         counterpart (256 random-token prompts of 100..1024 tokens, 100..1024 output tokens each,
+         temperature 0.6, no EOS): output tokens per second; --steps/--warmup are ignored.
   copy = a plain 1 GiB device-to-device tensor copy (not a mops op): the known-size kernel against which
          the FETCH_SIZE / WRITE_SIZE counters of a profile are calibrated.
 
@@ -31,10 +34,60 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding", "copy"])
+                    choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
+    ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
+    ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
+
+
+def run_e2e(args, torch, dev, mops):
+    """Workload of the reference's bench.py:9-28 on the engine counterpart, hip backend; plus a reduced
+    run of the same engine on the CPU-restated torch backend (on the GPU) as the comparison baseline."""
+    import random
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    random.seed(0)
+    n = args.e2e_seqs
+    prompts = [[random.randint(0, 10000) for _ in range(random.randint(100, 1024))] for _ in range(n)]
+    max_tokens = [random.randint(100, 1024) for _ in range(n)]
+    eng = Engine(Qwen3Shape(), backend="hip", num_blocks=max(64, n * 10), seed=args.seed)
+    eng.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 8)                 # warm-up, as the reference does
+    if not args.e2e_eager:
+        eng.capture_decode_graphs(max_bs=min(512, max(16, (n + 15) // 16 * 16)), max_model_len=4096)
+    _, st = eng.generate(prompts, max_tokens, temperature=0.6)
+    total = sum(max_tokens)
+    out = {
+        "metric": "e2e_output_tok_per_s", "value": round(total / st["total_s"], 2), "unit": "tok/s", "n_gpus": 1,
+        "steps": st["prefill_steps"] + st["decode_steps"], "warmup": 1,
+        "ms_per_step": round(st["total_s"] * 1e3 / (st["prefill_steps"] + st["decode_steps"]), 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg5 end-to-end generate, random-init Qwen3-0.6B architecture, mops hip backend, decode step "
+                               + ("eager" if args.e2e_eager else "replayed from HIP graphs"),
+                   "prompts": n, "prompt_len": "uniform[100,1024]", "max_tokens": "uniform[100,1024]", "temperature": 0.6,
+                   "output_tokens": total, "prompt_tokens": sum(len(p) for p in prompts)},
+        "breakdown": {"seconds": round(st["total_s"], 3), "prefill_steps": st["prefill_steps"], "decode_steps": st["decode_steps"],
+                      "prefill_tok_per_s": round(st["prefill_tokens"] / max(st["prefill_s"], 1e-9), 1),
+                      "decode_tok_per_s": round(st["decode_tokens"] / max(st["decode_s"], 1e-9), 1)},
+    }
+    if not args.no_cpu_baseline:
+        del eng
+        torch.cuda.empty_cache()
+        import oracle.mops_torch  # noqa: F401  comparison backend only
+        m, outlen = 16, 16
+        res = {}
+        for backend in ("hip", "torch"):
+            e = Engine(Qwen3Shape(), backend=backend, num_blocks=m * 6, seed=args.seed)
+            e.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 4)
+            _, s2 = e.generate(prompts[:m], outlen, temperature=0.6)
+            res[backend] = m * outlen / s2["total_s"]
+            del e
+            torch.cuda.empty_cache()
+        out["comparison_baseline"] = {"what": "same engine, same GPU, mops ops from the pure-torch restatement of the reference's torch "
+                                              "backend (per-sequence attention loops)", "sample": f"first {m} prompts, {outlen} output tokens each",
+                                      "hip_tok_per_s": round(res["hip"], 1), "torch_tok_per_s": round(res["torch"], 1),
+                                      "speedup": round(res["hip"] / res["torch"], 2)}
+    print(json.dumps(out))
 
 
 def main():
@@ -71,6 +124,10 @@ def main():
 
     cpu_fn = None      # () -> (seconds, description, units_done)  on a bounded sample
     measured_traffic = None
+
+    if args.op == "e2e":
+        run_e2e(args, torch, dev, mops)
+        return
     bound = "hbm"
     dtype = "bf16"
 

@@ -122,7 +122,7 @@ int mops_hip_add_rms_forward(const void* x, int64_t x_row_stride,
  * out: contiguous [batch, hq, 128] bf16.
  * workspace: device scratch of at least mops_hip_paged_decode_workspace_bytes(...) bytes, 256-byte
  * aligned, private to this call until it completes on `stream`.
- * Supported: head_dim 128, block_size a multiple of 32, hq/hkv in {1,2,4,8,16}.
+ * Supported: head_dim 128, block_size a multiple of 32, hq/hkv <= 16, num_blocks >= 1.
  */
 int64_t mops_hip_paged_decode_workspace_bytes(int64_t batch, int64_t hq, int64_t hkv,
                                               int64_t max_blocks_per_seq, int64_t block_size);
@@ -160,6 +160,27 @@ int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_stride,
                                      int64_t hq, int64_t hkv, int64_t head_dim,
                                      float softmax_scale,
                                      void* stream);
+
+/*
+ * siluAndMul — out = bf16( bf16(silu(x)) * y ), elementwise over [rows, n].
+ * Replaces: mops/torch/ops.py:32-34 (F.silu(x) * y), mops/ninetoothed/activation.py:10-32; called at
+ * nanovllm/layers/activation.py:16 with x, y the two halves of the gate_up projection (row strides in
+ * elements; out contiguous [rows, n]).  n % 8 == 0, strides % 8 == 0.
+ */
+int mops_hip_silu_and_mul(const void* x, int64_t x_row_stride, const void* y, int64_t y_row_stride,
+                          void* out, int64_t rows, int64_t n, void* stream);
+
+/*
+ * apply_rotary_emb — neox-style half-split rotation of x [tokens, heads, head_dim] bf16 by per-token
+ * fp32 cos/sin rows of head_dim/2 values: y1 = x1*cos - x2*sin, y2 = x2*cos + x1*sin (fp32, products
+ * rounded separately), out contiguous [tokens, heads, head_dim] bf16.
+ * Replaces: mops/torch/ops.py:45-54, mops/ninetoothed/rotary_emb.py:10-65; called at
+ * nanovllm/layers/rotary_embedding.py:35-36.  head_dim % 16 == 0.
+ */
+int mops_hip_apply_rotary_emb(const void* x, int64_t x_token_stride, int64_t x_head_stride,
+                              const float* cos, int64_t cos_token_stride,
+                              const float* sin, int64_t sin_token_stride,
+                              void* out, int64_t tokens, int64_t heads, int64_t head_dim, void* stream);
 
 #ifdef __cplusplus
 }

@@ -34,9 +34,12 @@ SIGNATURES = {
     "mops_hip_attn_varlen_causal_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                                  c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64,
                                                  c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "mops_hip_silu_and_mul": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
+    "mops_hip_apply_rotary_emb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
+                                          c_int64, c_int64, c_int64, c_void_p]),
 }
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 

@@ -1,5 +1,6 @@
-"""The `hip` backend: the six hot operators run hand-written gfx950 kernels through the C ABI of
-libmops_hip.so; the remaining names are library-torch delegates so that the engine's layers resolve.
+"""The `hip` backend: the six hot operators, plus siluAndMul and apply_rotary_emb, run hand-written gfx950
+kernels through the C ABI of libmops_hip.so; linear, sampler_forward and softmax are library-torch
+delegates so that the engine's layers resolve.
 
 Every function keeps the name and call form the reference's layers use (nanovllm/layers/attention.py:29-42,
 layernorm.py:21,29, embed_head.py:41).  Wrappers validate layouts with exceptions before launching
@@ -229,7 +230,8 @@ def flash_attn_varlen_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ma
 
 
 # ----------------------------------------------------------------------------------------------------
-# remaining registry names: library torch on the GPU, as in mops/torch/ops.py:5-7,32-54
+# remaining registry names: the two per-layer elementwise ops have kernels of their own; linear, sampler
+# and softmax are library torch on the GPU, as in mops/torch/ops.py:5-7,37-43
 # ----------------------------------------------------------------------------------------------------
 
 @register_hip_op
@@ -239,7 +241,23 @@ def linear(x, weight, bias=None):
 
 @register_hip_op
 def siluAndMul(x: torch.Tensor, y: torch.Tensor):
-    return torch.nn.functional.silu(x) * y
+    """silu(x) * y with the two bf16 roundings of the library expression (mops/torch/ops.py:32-34); x and y
+    are usually the two halves of one gate_up buffer and are read in place."""
+    _require_cuda_bf16("x", x)
+    _require_cuda_bf16("y", y)
+    _require(x.shape == y.shape, "x and y must have the same shape")
+    n = x.shape[-1]
+    x2, y2 = x.reshape(-1, n), y.reshape(-1, n)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    if y2.stride(1) != 1:
+        y2 = y2.contiguous()
+    rows = x2.shape[0]
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    st = _capi.load().mops_hip_silu_and_mul(x2.data_ptr(), x2.stride(0) if rows > 1 else n, y2.data_ptr(),
+                                            y2.stride(0) if rows > 1 else n, out.data_ptr(), rows, n, _stream(x))
+    _capi.check("mops_hip_silu_and_mul", st)
+    return out
 
 
 @register_hip_op
@@ -251,10 +269,20 @@ def sampler_forward(logits: torch.Tensor, temperatures: torch.Tensor):
 
 @register_hip_op
 def apply_rotary_emb(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    x1, x2 = torch.chunk(x.float(), 2, dim=-1)
-    y1 = x1 * cos - x2 * sin
-    y2 = x2 * cos + x1 * sin
-    return torch.cat((y1, y2), dim=-1).to(x.dtype)
+    """Half-split rotary embedding, x [T, H, D] bf16, cos/sin [T, 1, D/2] fp32 (mops/torch/ops.py:45-54)."""
+    _require_cuda_bf16("x", x)
+    _require(x.dim() == 3 and x.stride(2) == 1, "x must be [tokens, heads, head_dim] with contiguous head_dim")
+    t, h, d = x.shape
+    _require(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_cuda and sin.is_cuda, "cos/sin must be fp32 GPU tensors")
+    _require(cos.shape == sin.shape and cos.numel() == t * (d // 2) and cos.shape[-1] == d // 2 and cos.stride(-1) == 1
+             and sin.stride(-1) == 1, "cos/sin must be [tokens, 1, head_dim/2] with a contiguous last dim")
+    out = torch.empty((t, h, d), dtype=x.dtype, device=x.device)
+    st = _capi.load().mops_hip_apply_rotary_emb(x.data_ptr(), x.stride(0) if t > 1 else h * d, x.stride(1) if h > 1 else d,
+                                                cos.data_ptr(), cos.stride(0) if t > 1 else d // 2,
+                                                sin.data_ptr(), sin.stride(0) if t > 1 else d // 2,
+                                                out.data_ptr(), t, h, d, _stream(x))
+    _capi.check("mops_hip_apply_rotary_emb", st)
+    return out
 
 
 @register_hip_op

@@ -97,8 +97,8 @@ def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, cau
     vf = v.to(torch.float32).transpose(0, 1).repeat_interleave(rep, dim=0)
     scores = torch.matmul(qf, kf.transpose(1, 2)) * scale
     if causal_offset is not None:
-        i = torch.arange(lq).unsqueeze(1)
-        j = torch.arange(lk).unsqueeze(0)
+        i = torch.arange(lq, device=q.device).unsqueeze(1)
+        j = torch.arange(lk, device=q.device).unsqueeze(0)
         scores = scores.masked_fill(j > i + causal_offset, float("-inf"))
     probs = torch.softmax(scores, dim=-1)
     return torch.matmul(probs, vf).transpose(0, 1)                            # [Lq, Hq, D] fp32
