@@ -19,6 +19,13 @@
 //                                      already the B-operand layout, V^T comes out of LDS through
 //                                      ds_read_b64_tr_b16, also issued ahead of the MFMAs that use it
 //
+// What bounds this shape: on this part ds_read_b128 streams ~210 B/clk per CU, but the transposing read
+// ds_read_b64_tr_b16 only ~65 B/clk and ds_write_b128 ~73 B/clk (measured).  With 32 query rows per wave
+// every 32-cycle MFMA of the second product needs 1 KiB of V^T through the transposing read, so the
+// LDS pipe, not the matrix pipe, sets the pace (~58 % MFMA at best).  A wave owning 64 rows halves that
+// traffic but needs ~400 VGPRs, i.e. one wave per SIMD, and then only pays off with the two products
+// and the softmax software-pipelined across tiles inside the wave.
+//
 // LDS rows are padded instead of swizzled (K rows 272 B apart, V rows 320 B apart): the K operand read
 // (16 consecutive rows, one 16-byte piece) and the transposing V read (4 rows x 4 pieces) each cover
 // all 64 banks once, and every address a lane needs is one base register plus an immediate.
