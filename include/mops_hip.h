@@ -139,24 +139,33 @@ int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
                                     void* stream);
 
 /*
- * Varlen (packed, THD) causal prefill attention with grouped-query heads.
+ * Varlen (packed, THD) causal prefill attention with grouped-query heads, with or without a cached prefix.
  * Replaces: flash_attn.flash_attn_varlen_func as reached from mops/torch/ops.py:70-72 and the Triton
- * kernel mops/triton/attention.py:42-146; called at nanovllm/layers/attention.py:34-37.
+ * kernel mops/triton/attention.py:42-146; called at nanovllm/layers/attention.py:34-37 (with the paged
+ * caches as k/v and block_table set when a prefix-cache hit occurred, attention.py:32-33).
  *
- *   for sequence s with tokens [cu_seqlens[s], cu_seqlens[s+1]):
- *     out[i,h,:] = softmax_{j<=i}( scale * q[i,h,:] . k[j,h/(hq/hkv),:] ) @ v[j,h/(hq/hkv),:]
+ *   for sequence s with query tokens [cu_q[s], cu_q[s+1]) and Lk = cu_k[s+1]-cu_k[s] keys (Lk >= Lq):
+ *     out[i,h,:] = softmax_{j <= i + (Lk-Lq)}( scale * q[i,h,:] . K_s[j,h/(hq/hkv),:] ) @ V_s[j,h/(hq/hkv),:]
  *
- * q/k/v/out: [total_tokens, heads, 128] bf16 with per-tensor token strides (elements) and head stride
- * 128; cu_seqlens: int32 [batch+1], cu_seqlens[0] == 0, non-decreasing, last == total_tokens
- * (q and k share it: no prefix-cache path here).  max_seqlen bounds every sequence length and only
- * sizes the launch.  Sequences of length 0 are allowed.
+ * q/out: [total_tokens, hq, 128] bf16, token strides in elements, head stride 128.
+ * block_table == NULL: k/v are packed [total_k_tokens, hkv, 128] with their own token strides and key j of
+ *   sequence s is row cu_k[s] + j; cu_seqlens_k may be NULL (then it equals cu_seqlens_q).
+ * block_table != NULL: k/v are the contiguous paged caches [num_blocks, block_size, hkv, 128] and key j of
+ *   sequence s is cache[block_table[s, j/block_size], j%block_size] (row stride block_table_row_stride,
+ *   at least max_blocks_per_seq columns; entries beyond the sequence's keys are never read; block_size
+ *   must be a multiple of 64); k/v token strides are ignored.
+ * cu_seqlens_*: int32 [batch+1], non-decreasing, starting at 0.  max_seqlen_q bounds every query length
+ * and only sizes the launch.  Sequences of length 0 are allowed.
  */
 int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_stride,
                                      const void* k, int64_t k_token_stride,
                                      const void* v, int64_t v_token_stride,
                                      void* out, int64_t out_token_stride,
-                                     const int32_t* cu_seqlens,
-                                     int64_t batch, int64_t total_tokens, int64_t max_seqlen,
+                                     const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                     const int32_t* block_table, int64_t block_table_row_stride,
+                                     int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                     int64_t batch, int64_t total_tokens, int64_t total_k_tokens,
+                                     int64_t max_seqlen_q,
                                      int64_t hq, int64_t hkv, int64_t head_dim,
                                      float softmax_scale,
                                      void* stream);

@@ -32,14 +32,15 @@ SIGNATURES = {
                                                 c_int64, c_int64, c_int64, c_float, c_void_p, c_int64,
                                                 c_void_p]),
     "mops_hip_attn_varlen_causal_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
-                                                 c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64,
+                                                 c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64,
+                                                 c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                                  c_int64, c_int64, c_int64, c_float, c_void_p]),
     "mops_hip_silu_and_mul": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
     "mops_hip_apply_rotary_emb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p]),
 }
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 

@@ -49,8 +49,12 @@ struct PrefillParams {
   const uint16_t* v;
   uint16_t* out;
   int64_t q_ts, k_ts, v_ts, o_ts;  // token strides (elements)
-  const int32_t* cu_seqlens;
-  int batch, total_tokens, m_tiles, hq, hkv, group;
+  const int32_t* cu_seqlens;     // query side [batch+1]
+  const int32_t* cu_seqlens_k;   // key side [batch+1]; equal to cu_seqlens when there is no cached prefix
+  const int32_t* block_table;    // null: k/v are packed [total_k_tokens, hkv, 128]; else they are the paged caches
+  int64_t block_table_row_stride;
+  int block_size, num_blocks, max_blocks_per_seq;
+  int batch, total_tokens, total_k_tokens, m_tiles, hq, hkv, group;
   float scale_log2;
 };
 
@@ -84,9 +88,16 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   const int b = rest % p.batch;
   const int m = p.m_tiles - 1 - rest / p.batch;
   const int seq_begin = p.cu_seqlens[b];
-  const int seq_len = min(p.cu_seqlens[b + 1], p.total_tokens) - seq_begin;
+  const int seq_len = min(p.cu_seqlens[b + 1], p.total_tokens) - seq_begin;   // query rows of this sequence
   const int q0 = m * kPBM;
   if (seq_begin < 0 || q0 >= seq_len) return;
+  // keys of this sequence: kv_len >= seq_len when a cached prefix precedes the new tokens; query row i
+  // then sees keys 0 .. i + shift (bottom-right aligned causal mask)
+  const int kbegin = p.cu_seqlens_k[b];
+  int kv_len = p.cu_seqlens_k[b + 1] - kbegin;
+  const bool paged = p.block_table != nullptr;
+  kv_len = max(0, min(kv_len, paged ? p.max_blocks_per_seq * p.block_size : p.total_k_tokens - kbegin));
+  const int shift = kv_len - seq_len;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -95,13 +106,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   const int jj = lane >> 5;  // half: k slice / row-quad selector
   const int g = h / p.group;
 
-  const int kv_end = min(seq_len, q0 + kPBM);
+  const int kv_end = max(0, min(kv_len, q0 + kPBM + shift));
   const int ntiles = (kv_end + kPBN - 1) / kPBN;
   const int wave_row0 = q0 + 32 * wave;          // first q row (sequence-relative) of this wave
   const int my_row = wave_row0 + n;
-  // tiles this wave has to look at: those holding a key visible to one of its rows.  Only the last of
-  // them crosses the diagonal (or the end of the sequence) and needs the mask.
-  const int my_tiles = min(ntiles, (wave_row0 + 31) / kPBN + 1);
+  // tiles this wave has to look at: those holding a key visible to one of its rows
+  const int my_tiles = max(0, min(ntiles, (wave_row0 + 31 + shift >= 0) ? (wave_row0 + 31 + shift) / kPBN + 1 : 0));
 
   // ---- Q^T as B operand: lane (n, jj) holds Q[my_row][16*kb + 8*jj .. +8) for kb = 0..7
   bf16x8 qb[8];
@@ -119,19 +129,32 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   // ---- cooperative tile loads: thread moves 16-byte piece (tid & 15) of rows (tid >> 4) + 16*i
   const int ld_row = tid >> 4;
   const int ld_slice = tid & 15;
-  const uint16_t* kptr = p.k + (int64_t)(seq_begin + ld_row) * p.k_ts + (int64_t)g * kPD + (ld_slice << 3);
-  const uint16_t* vptr = p.v + (int64_t)(seq_begin + ld_row) * p.v_ts + (int64_t)g * kPD + (ld_slice << 3);
-  auto load_tile = [&](const uint16_t* base, int64_t ts, int tile, u32x4 (&r)[4]) {
-    const uint16_t* src = base + (int64_t)tile * kPBN * ts;
-    if ((tile + 1) * kPBN <= seq_len) {  // whole tile inside the sequence
+  const int64_t tok_elems = (int64_t)p.hkv * kPD;   // elements between tokens inside a cache block
+  const int col = g * kPD + (ld_slice << 3);
+  const uint16_t* kptr = p.k + (int64_t)(kbegin + ld_row) * p.k_ts + col;
+  const uint16_t* vptr = p.v + (int64_t)(kbegin + ld_row) * p.v_ts + col;
+  const int32_t* table = paged ? p.block_table + (int64_t)b * p.block_table_row_stride : nullptr;
+  auto load_tile = [&](const uint16_t* base, const uint16_t* cache, int64_t ts, int tile, u32x4 (&r)[4]) {
+    const uint16_t* src;
+    bool tile_ok = true;
+    if (paged) {  // a 64-token tile lies inside one cache block (block_size is a multiple of 64)
+      const int t0 = tile * kPBN;
+      const int blk = table[t0 / p.block_size];
+      tile_ok = blk >= 0 && blk < p.num_blocks;
+      src = cache + ((int64_t)(tile_ok ? blk : 0) * p.block_size + (t0 % p.block_size) + ld_row) * tok_elems + col;
+      ts = tok_elems;
+    } else {
+      src = base + (int64_t)tile * kPBN * ts;
+    }
+    if (tile_ok && (tile + 1) * kPBN <= kv_len) {  // whole tile inside the sequence
 #pragma unroll
       for (int i = 0; i < 4; ++i) r[i] = load16(src + (int64_t)(16 * i) * ts);
-    } else {                             // rows past the sequence read as zeros
+    } else {                                        // rows past the sequence read as zeros
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int t = tile * kPBN + ld_row + 16 * i;
         u32x4 x = {0u, 0u, 0u, 0u};
-        if (t < seq_len) x = load16(src + (int64_t)(16 * i) * ts);
+        if (tile_ok && t < kv_len) x = load16(src + (int64_t)(16 * i) * ts);
         r[i] = x;
       }
     }
@@ -192,7 +215,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
-          s[tt][r] = key <= my_row ? s[tt][r] : -INFINITY;
+          s[tt][r] = key <= my_row + shift ? s[tt][r] : -INFINITY;
         }
     }
     float m_loc = fmaxf(s[0][0], s[1][0]);
@@ -248,8 +271,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 
   // ---- tile loop: tile i+1 is in flight into registers while tile i is consumed out of LDS
   u32x4 kreg[4], vreg[4];
-  load_tile(kptr, p.k_ts, 0, kreg);
-  load_tile(vptr, p.v_ts, 0, vreg);
+  load_tile(kptr, p.k, p.k_ts, 0, kreg);
+  load_tile(vptr, p.v, p.v_ts, 0, vreg);
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
   f32x16 s[2];
@@ -259,12 +282,13 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     store_v(buf, vreg);
     __syncthreads();   // tile visible to all waves; the other buffer (tile-1) is free once everyone is here
     if (tile + 1 < ntiles) {
-      load_tile(kptr, p.k_ts, tile + 1, kreg);
-      load_tile(vptr, p.v_ts, tile + 1, vreg);
+      load_tile(kptr, p.k, p.k_ts, tile + 1, kreg);
+      load_tile(vptr, p.v, p.v_ts, tile + 1, vreg);
     }
     if (tile < my_tiles) {
       qk_tile(buf, s);
-      if (tile + 1 == my_tiles) softmax_pv(s, buf, tile * kPBN, std::true_type{});
+      // the mask is only needed where the tile holds a key beyond the first row's horizon
+      if (tile * kPBN + kPBN - 1 > wave_row0 + shift) softmax_pv(s, buf, tile * kPBN, std::true_type{});
       else softmax_pv(s, buf, tile * kPBN, std::false_type{});
     }
   }
@@ -291,25 +315,36 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
                                                 const void* k, int64_t k_token_stride,
                                                 const void* v, int64_t v_token_stride,
                                                 void* out, int64_t out_token_stride,
-                                                const int32_t* cu_seqlens,
-                                                int64_t batch, int64_t total_tokens, int64_t max_seqlen,
+                                                const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                                const int32_t* block_table, int64_t block_table_row_stride,
+                                                int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                                int64_t batch, int64_t total_tokens, int64_t total_k_tokens,
+                                                int64_t max_seqlen_q,
                                                 int64_t hq, int64_t hkv, int64_t head_dim,
                                                 float softmax_scale,
                                                 void* stream) {
   using namespace mops;
-  if (batch < 0 || total_tokens < 0 || max_seqlen < 0 || hq <= 0 || hkv <= 0) return MOPS_HIP_EINVAL;
-  if (batch == 0 || total_tokens == 0 || max_seqlen == 0) return MOPS_HIP_OK;
-  if (!q || !k || !v || !out || !cu_seqlens) return MOPS_HIP_EINVAL;
+  if (batch < 0 || total_tokens < 0 || total_k_tokens < 0 || max_seqlen_q < 0 || hq <= 0 || hkv <= 0) return MOPS_HIP_EINVAL;
+  if (batch == 0 || total_tokens == 0 || max_seqlen_q == 0) return MOPS_HIP_OK;
+  if (!q || !k || !v || !out || !cu_seqlens_q) return MOPS_HIP_EINVAL;
   if (hq % hkv != 0) return MOPS_HIP_EINVAL;
   if (head_dim != kPD) return MOPS_HIP_EUNSUPPORTED;
-  if (q_token_stride < hq * kPD || out_token_stride < hq * kPD || k_token_stride < hkv * kPD ||
-      v_token_stride < hkv * kPD)
-    return MOPS_HIP_EINVAL;
-  if (total_tokens > 0x3fffffffLL || batch > (1 << 20) || hq > 4096) return MOPS_HIP_EUNSUPPORTED;
-  if ((q_token_stride & 7) || (k_token_stride & 7) || (v_token_stride & 7) || (out_token_stride & 3))
-    return MOPS_HIP_EALIGN;
+  if (q_token_stride < hq * kPD || out_token_stride < hq * kPD) return MOPS_HIP_EINVAL;
+  if (total_tokens > 0x3fffffffLL || total_k_tokens > 0x3fffffffLL || batch > (1 << 20) || hq > 4096) return MOPS_HIP_EUNSUPPORTED;
+  if ((q_token_stride & 7) || (out_token_stride & 3)) return MOPS_HIP_EALIGN;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return MOPS_HIP_EALIGN;
-  if (max_seqlen > total_tokens) max_seqlen = total_tokens;
+  if (block_table) {
+    if (!cu_seqlens_k || block_size <= 0 || num_blocks <= 0 || max_blocks_per_seq <= 0 ||
+        block_table_row_stride < max_blocks_per_seq)
+      return MOPS_HIP_EINVAL;
+    if (block_size % kPBN != 0 || num_blocks * block_size > (int64_t)0x7fffffff || max_blocks_per_seq * block_size > (1 << 24))
+      return MOPS_HIP_EUNSUPPORTED;
+  } else {
+    if (k_token_stride < hkv * kPD || v_token_stride < hkv * kPD) return MOPS_HIP_EINVAL;
+    if ((k_token_stride & 7) || (v_token_stride & 7)) return MOPS_HIP_EALIGN;
+    if (!cu_seqlens_k && total_k_tokens != total_tokens) return MOPS_HIP_EINVAL;
+  }
+  if (max_seqlen_q > total_tokens) max_seqlen_q = total_tokens;
 
   PrefillParams p;
   p.q = (const uint16_t*)q;
@@ -320,10 +355,17 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   p.k_ts = k_token_stride;
   p.v_ts = v_token_stride;
   p.o_ts = out_token_stride;
-  p.cu_seqlens = cu_seqlens;
+  p.cu_seqlens = cu_seqlens_q;
+  p.cu_seqlens_k = cu_seqlens_k ? cu_seqlens_k : cu_seqlens_q;
+  p.block_table = block_table;
+  p.block_table_row_stride = block_table_row_stride;
+  p.block_size = (int)block_size;
+  p.num_blocks = (int)num_blocks;
+  p.max_blocks_per_seq = (int)max_blocks_per_seq;
   p.batch = (int)batch;
   p.total_tokens = (int)total_tokens;
-  p.m_tiles = (int)((max_seqlen + kPBM - 1) / kPBM);
+  p.total_k_tokens = (int)total_k_tokens;
+  p.m_tiles = (int)((max_seqlen_q + kPBM - 1) / kPBM);
   p.hq = (int)hq;
   p.hkv = (int)hkv;
   p.group = (int)(hq / hkv);

@@ -200,31 +200,53 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 def flash_attn_varlen_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, max_seqlen_q=None, cu_seqlens_q=None,
                            max_seqlen_k=None, cu_seqlens_k=None, softmax_scale=None, causal=True, block_table=None,
                            **kwargs) -> torch.Tensor:
-    """Varlen causal prefill attention over packed [T, H, D] tensors (call form: nanovllm/layers/attention.py:34-37)."""
+    """Varlen causal prefill attention over packed [T, H, D] queries (call form: nanovllm/layers/attention.py:34-37).
+    With block_table given, k and v are the paged caches and each sequence's keys are its cu_seqlens_k span
+    (cached prefix + new tokens), masked bottom-right aligned."""
     _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
-    if block_table is not None:
-        raise NotImplementedError("prefix-cache prefill (block_table given) is not implemented by the hip backend")
     _require(causal, "only causal attention is implemented")
     _require(cu_seqlens_q is not None and max_seqlen_q is not None, "cu_seqlens_q and max_seqlen_q are required")
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        _require_cuda_bf16(name, t)
-        _require(t.dim() == 3 and t.stride(2) == 1 and t.stride(1) == t.shape[2], f"{name} must be [T, H, D] with contiguous heads")
+    _require_cuda_bf16("q", q)
+    _require(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [T, H, D] with contiguous heads")
     total, hq, d = q.shape
-    _require(k.shape == v.shape and k.shape[0] == total and k.shape[2] == d, "k/v must be [T, Hkv, D] matching q")
-    hkv = k.shape[1]
-    _require(hq % hkv == 0, "query heads must be a multiple of kv heads")
     _require(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_cuda and cu_seqlens_q.is_contiguous(),
              "cu_seqlens_q must be a contiguous int32 GPU tensor")
-    if cu_seqlens_k is not None and cu_seqlens_k is not cu_seqlens_q:
-        _require(cu_seqlens_k.shape == cu_seqlens_q.shape, "cu_seqlens_k must match cu_seqlens_q (no prefix cache)")
     batch = cu_seqlens_q.numel() - 1
+    if cu_seqlens_k is not None:
+        _require(cu_seqlens_k.dtype == torch.int32 and cu_seqlens_k.is_cuda and cu_seqlens_k.is_contiguous()
+                 and cu_seqlens_k.shape == cu_seqlens_q.shape, "cu_seqlens_k must be an int32 GPU tensor shaped like cu_seqlens_q")
     scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(d)
     out = torch.empty((total, hq, d), dtype=q.dtype, device=q.device)
     lib = _capi.load()
-    ts = lambda t, h: t.stride(0) if total > 1 else h * d  # noqa: E731
-    st = lib.mops_hip_attn_varlen_causal_bf16(q.data_ptr(), ts(q, hq), k.data_ptr(), ts(k, hkv), v.data_ptr(),
-                                              ts(v, hkv), out.data_ptr(), hq * d, cu_seqlens_q.data_ptr(), batch,
-                                              total, int(max_seqlen_q), hq, hkv, d, scale, _stream(q))
+    cu_k_ptr = cu_seqlens_k.data_ptr() if cu_seqlens_k is not None else None
+    if block_table is None:
+        for name, t in (("k", k), ("v", v)):
+            _require_cuda_bf16(name, t)
+            _require(t.dim() == 3 and t.stride(2) == 1 and t.stride(1) == t.shape[2], f"{name} must be [T, H, D] with contiguous heads")
+        _require(k.shape == v.shape and k.shape[2] == d, "k/v must be [Tk, Hkv, D] matching q's head_dim")
+        total_k, hkv = k.shape[0], k.shape[1]
+        _require(cu_seqlens_k is not None or total_k == total, "k/v must have as many tokens as q when cu_seqlens_k is not given")
+        ks = k.stride(0) if total_k > 1 else hkv * d
+        vs = v.stride(0) if total_k > 1 else hkv * d
+        bt_ptr, bt_stride, bs, nblk, maxblk = None, 0, 0, 0, 0
+    else:
+        _require(cu_seqlens_k is not None, "cu_seqlens_k is required with block_table")
+        for name, t in (("k_cache", k), ("v_cache", v)):
+            _require_cuda_bf16(name, t)
+            _require(t.dim() == 4 and t.is_contiguous() and t.shape[3] == d, f"{name} must be a contiguous [blocks, block_size, kv_heads, D] cache")
+        _require(k.shape == v.shape, "k_cache and v_cache must have the same shape")
+        nblk, bs, hkv, _ = k.shape
+        _require(block_table.dtype == torch.int32 and block_table.is_cuda and block_table.dim() == 2
+                 and block_table.shape[0] == batch and block_table.stride(1) == 1,
+                 "block_table must be an int32 GPU tensor [batch, max_blocks] with contiguous rows")
+        maxblk = block_table.shape[1]
+        bt_ptr, bt_stride = block_table.data_ptr(), (block_table.stride(0) if batch > 1 else maxblk)
+        total_k, ks, vs = 0, 0, 0
+    _require(hq % hkv == 0, "query heads must be a multiple of kv heads")
+    st = lib.mops_hip_attn_varlen_causal_bf16(q.data_ptr(), q.stride(0) if total > 1 else hq * d, k.data_ptr(), ks,
+                                              v.data_ptr(), vs, out.data_ptr(), hq * d, cu_seqlens_q.data_ptr(), cu_k_ptr,
+                                              bt_ptr, bt_stride, bs, nblk, maxblk, batch, total, total_k, int(max_seqlen_q),
+                                              hq, hkv, d, scale, _stream(q))
     _capi.check("mops_hip_attn_varlen_causal_bf16", st)
     return out
 

@@ -77,6 +77,44 @@ def prefill_inputs(seq_lens, hq: int = 16, hkv: int = 8, seed: int = 0) -> dict:
     }
 
 
+def prefix_prefill_inputs(new_lens, prefix_lens, hq: int = 16, hkv: int = 8, seed: int = 0, poison_unused: bool = True) -> dict:
+    """Prefill with a cached prefix (the prefix-cache hit path): sequence s has prefix_lens[s] tokens already
+    in the paged cache followed by new_lens[s] new ones whose K/V have just been stored there too; q holds
+    only the new tokens.  Returns the paged caches, block_table, cu_seqlens_q/k and, for checking, the
+    packed K/V of every sequence."""
+    g = _gen(seed)
+    new = torch.as_tensor(new_lens, dtype=torch.int64)
+    tot = new + torch.as_tensor(prefix_lens, dtype=torch.int64)
+    bsz = len(new)
+    blocks_per_seq = (tot + BLOCK_SIZE - 1) // BLOCK_SIZE
+    nblk = int(blocks_per_seq.sum()) + 2
+    max_blocks = max(int(blocks_per_seq.max()), 1)
+    perm = torch.randperm(nblk, generator=g).to(torch.int32)
+    table = torch.full((bsz, max_blocks), -1, dtype=torch.int32)
+    fill = float("nan") if poison_unused else 0.0
+    k_cache = torch.full((nblk, BLOCK_SIZE, hkv, HEAD_DIM), fill, dtype=torch.bfloat16)
+    v_cache = torch.full((nblk, BLOCK_SIZE, hkv, HEAD_DIM), fill, dtype=torch.bfloat16)
+    k_all = _normal(g, (int(tot.sum()), hkv, HEAD_DIM))
+    v_all = _normal(g, (int(tot.sum()), hkv, HEAD_DIM))
+    cu_q = torch.zeros(bsz + 1, dtype=torch.int32)
+    cu_k = torch.zeros(bsz + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(new, 0).to(torch.int32)
+    cu_k[1:] = torch.cumsum(tot, 0).to(torch.int32)
+    pos = 0
+    for b in range(bsz):
+        nb = int(blocks_per_seq[b])
+        table[b, :nb] = perm[pos:pos + nb]
+        pos += nb
+        lo = int(cu_k[b])
+        for i in range(nb):
+            n = min(BLOCK_SIZE, int(tot[b]) - i * BLOCK_SIZE)
+            k_cache[int(table[b, i]), :n] = k_all[lo + i * BLOCK_SIZE: lo + i * BLOCK_SIZE + n]
+            v_cache[int(table[b, i]), :n] = v_all[lo + i * BLOCK_SIZE: lo + i * BLOCK_SIZE + n]
+    return {"q": _normal(g, (int(new.sum()), hq, HEAD_DIM)), "k_cache": k_cache, "v_cache": v_cache, "k_all": k_all, "v_all": v_all,
+            "cu_seqlens_q": cu_q, "cu_seqlens_k": cu_k, "block_table": table, "max_seqlen_q": int(new.max()),
+            "max_seqlen_k": int(tot.max()), "scale": HEAD_DIM ** -0.5}
+
+
 def prefill_flops(seq_lens, hq: int = 16) -> float:
     """Causal attention flops: two products of 2*D flops per (query, visible key, head)."""
     return float(sum(4 * HEAD_DIM * hq * l * (l + 1) // 2 for l in seq_lens))

@@ -41,6 +41,23 @@ def varlen_causal(q: np.ndarray, k: np.ndarray, v: np.ndarray, cu_seqlens, scale
     return out
 
 
+def varlen_causal_prefix(q: np.ndarray, k: np.ndarray, v: np.ndarray, cu_q, cu_k, scale: float) -> np.ndarray:
+    """As varlen_causal, but sequence s has Lk >= Lq keys (k/v packed by cu_k): its query i, counted from
+    the first NEW token, sits at absolute position i + (Lk - Lq) and sees the keys at positions <= that."""
+    T, Hq, D = q.shape
+    rep = Hq // k.shape[1]
+    out = np.zeros((T, Hq, D), dtype=np.float64)
+    for s in range(len(cu_q) - 1):
+        q_lo, q_hi, k_lo, k_hi = int(cu_q[s]), int(cu_q[s + 1]), int(cu_k[s]), int(cu_k[s + 1])
+        first_new = (k_hi - k_lo) - (q_hi - q_lo)
+        for i in range(q_hi - q_lo):
+            last_visible = first_new + i
+            for h in range(Hq):
+                out[q_lo + i, h] = attention_row(q[q_lo + i, h], k[k_lo:k_lo + last_visible + 1, h // rep],
+                                                 v[k_lo:k_lo + last_visible + 1, h // rep], scale)
+    return out
+
+
 def paged_decode(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, cache_seqlens, block_table,
                  scale: float) -> np.ndarray:
     """q [B,Hq,D]; caches [NB,BS,Hkv,D]; token t of sequence b is cache[block_table[b][t // BS], t % BS]."""

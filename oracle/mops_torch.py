@@ -108,18 +108,28 @@ def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, cau
 def flash_attn_varlen_func(q, k, v, max_seqlen_q=None, cu_seqlens_q=None, max_seqlen_k=None, cu_seqlens_k=None,
                            softmax_scale=None, causal=True, block_table=None, **kwargs):
     """Packed causal attention, semantics of flash_attn.flash_attn_varlen_func as used at
-    nanovllm/layers/attention.py:34-37 and restated by mops/triton/attention.py:59-102,110-146."""
-    assert block_table is None, "prefix-cache prefill is outside the oracle"
+    nanovllm/layers/attention.py:34-37 and restated by mops/triton/attention.py:59-102,110-146.  When a
+    sequence has more keys than queries (cached prefix), the causal mask is aligned to the bottom right:
+    query i sees keys 0 .. i + (Lk - Lq)."""
     if cu_seqlens_k is None:
         cu_seqlens_k = cu_seqlens_q
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])
-    out = torch.empty_like(q)
+    out = torch.zeros_like(q)
     cq = cu_seqlens_q.tolist()
     ck = cu_seqlens_k.tolist()
     for s in range(len(cq) - 1):
-        qs, ks, vs = q[cq[s]:cq[s + 1]], k[ck[s]:ck[s + 1]], v[ck[s]:ck[s + 1]]
-        if qs.shape[0] == 0:
+        qs = q[cq[s]:cq[s + 1]]
+        n_k = ck[s + 1] - ck[s]
+        if qs.shape[0] == 0 or n_k <= 0:
             continue
+        if block_table is None:
+            ks, vs = k[ck[s]:ck[s + 1]], v[ck[s]:ck[s + 1]]
+        else:   # k, v are the paged caches (nanovllm/layers/attention.py:32-33): gather this sequence's keys
+            bs = k.shape[1]
+            nblk = (n_k + bs - 1) // bs
+            blocks = block_table[s, :nblk].long()
+            ks = k[blocks].reshape(nblk * bs, *k.shape[2:])[:n_k]
+            vs = v[blocks].reshape(nblk * bs, *v.shape[2:])[:n_k]
         off = (ks.shape[0] - qs.shape[0]) if causal else None
         out[cq[s]:cq[s + 1]] = _attend(qs, ks, vs, scale, off).to(q.dtype)
     return out

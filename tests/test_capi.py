@@ -81,15 +81,21 @@ def test_host_side_argument_validation(lib):
     assert decode(b=0) == 0
     # varlen prefill
     def prefill(**kw):
-        a = dict(q=A, qs=2048, k=A, ks=1024, v=A, vs=4096, o=A, os=2048, cu=A, b=2, t=512, ms=256, hq=16, hkv=8, d=128)
+        a = dict(q=A, qs=2048, k=A, ks=1024, v=A, vs=4096, o=A, os=2048, cu=A, cuk=None, bt=None, bts=0, bs=0, nb=0, mb=0,
+                 b=2, t=512, tk=512, ms=256, hq=16, hkv=8, d=128)
         a.update(kw)
         return lib.mops_hip_attn_varlen_causal_bf16(a["q"], a["qs"], a["k"], a["ks"], a["v"], a["vs"], a["o"], a["os"],
-                                                    a["cu"], a["b"], a["t"], a["ms"], a["hq"], a["hkv"], a["d"], 0.088, None)
+                                                    a["cu"], a["cuk"], a["bt"], a["bts"], a["bs"], a["nb"], a["mb"],
+                                                    a["b"], a["t"], a["tk"], a["ms"], a["hq"], a["hkv"], a["d"], 0.088, None)
     assert prefill(d=64) == -2
     assert prefill(cu=None) == -1
     assert prefill(ks=512) == -1
     assert prefill(vs=4100) == -3
     assert prefill(hq=12) == -1
+    assert prefill(tk=600) == -1                               # more keys than queries needs cu_seqlens_k
+    assert prefill(bt=A, bts=4, bs=256, nb=8, mb=4) == -1      # paged form needs cu_seqlens_k
+    assert prefill(bt=A, cuk=A, bts=2, bs=256, nb=8, mb=4) == -1   # table rows narrower than max_blocks
+    assert prefill(bt=A, cuk=A, bts=4, bs=96, nb=8, mb=4) == -2    # block size not a multiple of 64
     assert prefill(t=0) == 0
 
 

@@ -82,13 +82,48 @@ def test_prefill_empty_sequence_in_batch_and_no_tokens(gpu, ops):
     assert out.shape == (0, 16, 128)
 
 
-def test_prefill_rejects_prefix_cache_and_non_causal(gpu, ops):
+def test_prefill_rejects_non_causal(gpu, ops):
     hip, _ = ops("flash_attn_varlen_func")
     d = W.prefill_inputs([32], seed=29)
-    with pytest.raises(NotImplementedError):
-        _run(hip, d, gpu, block_table=torch.zeros((1, 1), dtype=torch.int32, device=gpu))
     with pytest.raises(ValueError):
         _run(hip, d, gpu, causal=False)
+
+
+def _run_prefix(op, d, dev, paged=True):
+    g = W.to_device(d, dev) if dev is not None else d
+    k, v = (g["k_cache"], g["v_cache"]) if paged else (g["k_all"], g["v_all"])
+    return op(g["q"], k, v, max_seqlen_q=d["max_seqlen_q"], cu_seqlens_q=g["cu_seqlens_q"], max_seqlen_k=d["max_seqlen_k"],
+              cu_seqlens_k=g["cu_seqlens_k"], softmax_scale=d["scale"], causal=True, block_table=g["block_table"] if paged else None)
+
+
+@pytest.mark.parametrize("new,prefix,hq,hkv", [
+    ([100, 200], [256, 512], 16, 8), ([1, 1, 1], [256, 1, 1023], 16, 8), ([300, 17, 129], [0, 256, 768], 16, 8),
+    ([64, 65], [63, 700], 32, 8), ([513], [1024], 8, 8), ([250, 5], [300, 2000], 8, 1)])
+def test_prefill_with_cached_prefix_matches_oracle(gpu, ops, new, prefix, hq, hkv):
+    """Prefix-cache hit (nanovllm/layers/attention.py:32-33 of the reference): k/v are the paged caches, keys
+    are addressed through block_table, causal mask aligned bottom-right; unused cache rows are NaN."""
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefix_prefill_inputs(new, prefix, hq=hq, hkv=hkv, seed=sum(new) + sum(prefix))
+    want = ref(d["q"], torch.nan_to_num(d["k_cache"]), torch.nan_to_num(d["v_cache"]), max_seqlen_q=d["max_seqlen_q"],
+               cu_seqlens_q=d["cu_seqlens_q"], max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"],
+               softmax_scale=d["scale"], causal=True, block_table=d["block_table"])
+    got = _run_prefix(hip, d, gpu, paged=True)
+    assert_attention_close(got, want, f"paged prefix prefill new={new} prefix={prefix}")
+    got_packed = _run_prefix(hip, d, gpu, paged=False)       # same keys handed over packed, with cu_seqlens_k
+    assert_bit_exact(got_packed, got, "packed keys with cu_seqlens_k vs paged keys")
+
+
+def test_prefix_prefill_last_row_equals_decode(gpu, ops):
+    pre, _ = ops("flash_attn_varlen_func")
+    dec, _ = ops("flash_attn_with_kvcache")
+    d = W.prefix_prefill_inputs([40, 7], [512, 300], seed=33, poison_unused=False)
+    g = W.to_device(d, gpu)
+    o = _run_prefix(pre, d, gpu)
+    last = (d["cu_seqlens_q"][1:] - 1).long()
+    lens = (d["cu_seqlens_k"][1:] - d["cu_seqlens_k"][:-1]).to(torch.int32)
+    od = dec(g["q"][last.to(gpu)].unsqueeze(1), g["k_cache"], g["v_cache"], cache_seqlens=lens.to(gpu), block_table=g["block_table"],
+             softmax_scale=d["scale"], causal=True)
+    assert_attention_close(od[:, 0], o[last.to(gpu)], "last new token vs a decode step over the same cache")
 
 
 def test_prefill_warmup_shape(gpu, ops):

@@ -194,3 +194,25 @@ def test_decode_invariants(O):
     assert (_decode(O, d0).float() == 0).all(), "empty context -> zeros"
     d1 = dict(d, cache_seqlens=torch.tensor([1], dtype=torch.int32))
     assert_bit_exact(_decode(O, d1)[0, 0], vc[1, 0].repeat_interleave(2, dim=0), "one cached token -> o = v")
+
+
+def test_prefix_prefill_against_fp64_brute_force_and_packed_form(O):
+    """Cached-prefix path: the paged form (caches + block_table) must equal the packed form (k/v spans by
+    cu_seqlens_k), and both the fp64 loops; with an empty prefix it reduces to plain causal prefill."""
+    d = W.prefix_prefill_inputs([5, 3, 7], [256, 0, 300], hq=4, hkv=2, seed=3)
+    paged = O.flash_attn_varlen_func(d["q"], d["k_cache"], d["v_cache"], max_seqlen_q=d["max_seqlen_q"], cu_seqlens_q=d["cu_seqlens_q"],
+                                     max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"], softmax_scale=d["scale"],
+                                     causal=True, block_table=d["block_table"])
+    packed = O.flash_attn_varlen_func(d["q"], d["k_all"], d["v_all"], max_seqlen_q=d["max_seqlen_q"], cu_seqlens_q=d["cu_seqlens_q"],
+                                      max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"], softmax_scale=d["scale"], causal=True)
+    assert torch.isfinite(paged.float()).all(), "NaN-poisoned unused cache rows must not reach the output"
+    assert_bit_exact(paged, packed, "paged vs packed keys")
+    want = BF.varlen_causal_prefix(d["q"].float().numpy(), d["k_all"].float().numpy(), d["v_all"].float().numpy(),
+                                   d["cu_seqlens_q"].tolist(), d["cu_seqlens_k"].tolist(), d["scale"])
+    assert np.abs(paged.float().numpy() - want).max() <= np.abs(want).max() * 2.0 ** -8 + 1e-6
+    # sequence 1 has no prefix: equals ordinary causal prefill of its 3 tokens
+    lo, hi = 5, 8
+    klo = int(d["cu_seqlens_k"][1])
+    plain = O.flash_attn_varlen_func(d["q"][lo:hi], d["k_all"][klo:klo + 3], d["v_all"][klo:klo + 3], max_seqlen_q=3,
+                                     cu_seqlens_q=torch.tensor([0, 3], dtype=torch.int32), softmax_scale=d["scale"], causal=True)
+    assert_bit_exact(paged[lo:hi], plain, "empty prefix")
