@@ -191,6 +191,16 @@ int mops_hip_apply_rotary_emb(const void* x, int64_t x_token_stride, int64_t x_h
                               const float* sin, int64_t sin_token_stride,
                               void* out, int64_t tokens, int64_t heads, int64_t head_dim, void* stream);
 
+/*
+ * sampler_forward — out[r] = argmax(softmax(logits[r, :] / temperature[r])) for positive temperatures, i.e.
+ * the index of the row's largest logit (first index on ties).  The temperatures do not change the result
+ * and are not passed.  Replaces: mops/torch/ops.py:37-43 (greedy: the Gumbel line is commented out),
+ * mops/ninetoothed/sampler_forward.py:9-94; called at nanovllm/layers/sampler.py:12.
+ * logits: [rows, n] bf16 with row stride in elements (% 8 == 0); out: int64 [rows].
+ */
+int mops_hip_sampler_argmax(const void* logits, int64_t row_stride, int64_t* out, int64_t rows, int64_t n,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif

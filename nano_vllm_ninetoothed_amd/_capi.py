@@ -38,9 +38,10 @@ SIGNATURES = {
     "mops_hip_silu_and_mul": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
     "mops_hip_apply_rotary_emb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p]),
+    "mops_hip_sampler_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
 }
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 

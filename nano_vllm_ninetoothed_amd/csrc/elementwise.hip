@@ -126,3 +126,70 @@ extern "C" int mops_hip_apply_rotary_emb(const void* x, int64_t x_token_stride, 
                      (uint16_t*)out, tokens, (int)heads, (int)half);
   return finish_launch();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// sampler_forward: token = argmax(softmax(logits / T)) per row (the reference's sampler is greedy: its
+// Gumbel line is commented out, mops/torch/ops.py:37-43).  Dividing by a positive temperature and
+// applying softmax are monotonic, so this is the index of the row's largest logit; the first such index
+// on ties, as torch.argmax returns.  One workgroup per row streams the row once.
+// ---------------------------------------------------------------------------------------------------
+namespace mops {
+
+constexpr int kArgmaxThreads = 1024;
+
+__global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16_t* __restrict__ logits, int64_t row_stride,
+                                                                   int64_t* __restrict__ out, int n) {
+  __shared__ float best_v[kArgmaxThreads / kWave];
+  __shared__ int best_i[kArgmaxThreads / kWave];
+  const uint16_t* row = logits + (int64_t)blockIdx.x * row_stride;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  const int pieces = n >> 3;
+  for (int pc = threadIdx.x; pc < pieces; pc += kArgmaxThreads) {
+    const u32x4 w = load16_stream(row + (pc << 3));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float lo = bf16lo_to_f32(w[e]), hi = bf16hi_to_f32(w[e]);
+      const int i0 = (pc << 3) + 2 * e;
+      if (lo > bv) { bv = lo; bi = i0; }        // strictly greater: within a lane indices only grow
+      if (hi > bv) { bv = hi; bi = i0 + 1; }
+    }
+  }
+  for (int i = (pieces << 3) + threadIdx.x; i < n; i += kArgmaxThreads) {  // tail when n % 8 != 0
+    const float x = bf16lo_to_f32(row[i]);
+    if (x > bv) { bv = x; bi = i; }
+  }
+  // NaN never compares greater; a row of NaNs yields index 0 like an all -inf row would
+#pragma unroll
+  for (int off = kWave / 2; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const int oi = __shfl_xor(bi, off, kWave);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    best_v[threadIdx.x / kWave] = bv;
+    best_i[threadIdx.x / kWave] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kArgmaxThreads / kWave; ++w)
+      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
+    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+}  // namespace mops
+
+extern "C" int mops_hip_sampler_argmax(const void* logits, int64_t row_stride, int64_t* out, int64_t rows, int64_t n,
+                                       void* stream) {
+  using namespace mops;
+  if (rows < 0 || n <= 0) return MOPS_HIP_EINVAL;
+  if (rows == 0) return MOPS_HIP_OK;
+  if (!logits || !out) return MOPS_HIP_EINVAL;
+  if (row_stride < n) return MOPS_HIP_EINVAL;
+  if (n > 0x7ffffff0LL || rows > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
+  if ((row_stride & 7) || !aligned16(logits)) return MOPS_HIP_EALIGN;
+  hipLaunchKernelGGL(row_argmax_kernel, dim3((unsigned)rows), dim3(kArgmaxThreads), 0, (hipStream_t)stream,
+                     (const uint16_t*)logits, row_stride, out, (int)n);
+  return finish_launch();
+}

@@ -531,6 +531,8 @@ extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_st
   if (batch >= (1 << 20) || hq > 4096 || hkv > 1024 || max_blocks_per_seq * block_size > (1 << 24) ||
       num_blocks * block_size > (int64_t)0x7fffffff)
     return MOPS_HIP_EUNSUPPORTED;
+  // the flat split counts 32-token stages in int32
+  if (batch * ((max_blocks_per_seq * block_size + kStageTokens - 1) / kStageTokens) > (int64_t)0x7fffffff) return MOPS_HIP_EUNSUPPORTED;
   if ((q_batch_stride & 7)) return MOPS_HIP_EALIGN;
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out)) return MOPS_HIP_EALIGN;
   hipStream_t s = (hipStream_t)stream;

@@ -1,5 +1,5 @@
-"""The `hip` backend: the six hot operators, plus siluAndMul and apply_rotary_emb, run hand-written gfx950
-kernels through the C ABI of libmops_hip.so; linear, sampler_forward and softmax are library-torch
+"""The `hip` backend: the six hot operators, plus siluAndMul, apply_rotary_emb and sampler_forward, run
+hand-written gfx950 kernels through the C ABI of libmops_hip.so; linear and softmax are library-torch
 delegates so that the engine's layers resolve.
 
 Every function keeps the name and call form the reference's layers use (nanovllm/layers/attention.py:29-42,
@@ -284,9 +284,19 @@ def siluAndMul(x: torch.Tensor, y: torch.Tensor):
 
 @register_hip_op
 def sampler_forward(logits: torch.Tensor, temperatures: torch.Tensor):
-    logits = logits.float().div_(temperatures.unsqueeze(dim=1))
-    probs = torch.softmax(logits, dim=-1)
-    return torch.argmax(probs, dim=-1)
+    """argmax(softmax(logits / T)) per row -> int64 [B] (mops/torch/ops.py:37-43; the reference samples
+    greedily).  For positive temperatures that is the index of the largest logit, computed in one pass
+    over the bf16 logits; other dtypes and layouts take the library expression."""
+    if logits.is_cuda and logits.dtype == torch.bfloat16 and logits.dim() == 2 and logits.stride(1) == 1 \
+            and logits.stride(0) % 8 == 0 and logits.data_ptr() % 16 == 0:
+        rows, n = logits.shape
+        out = torch.empty((rows,), dtype=torch.int64, device=logits.device)
+        st = _capi.load().mops_hip_sampler_argmax(logits.data_ptr(), logits.stride(0) if rows > 1 else max(n, (n + 7) // 8 * 8),
+                                                  out.data_ptr(), rows, n, _stream(logits))
+        _capi.check("mops_hip_sampler_argmax", st)
+        return out
+    scaled = logits.float().div_(temperatures.unsqueeze(dim=1))
+    return torch.argmax(torch.softmax(scaled, dim=-1), dim=-1)
 
 
 @register_hip_op

@@ -48,3 +48,23 @@ def test_silu_and_mul_matches_oracle(gpu, ops, rows, n):
     got = hip(xg, yg)
     assert got.shape == (rows, n) and got.is_contiguous()
     assert_rms_parity(got, torch.nn.functional.silu(x), y, want, "siluAndMul")
+
+
+@pytest.mark.parametrize("rows,vocab", [(256, 151936), (1, 151936), (7, 1000), (33, 2048), (5, 12345)])
+def test_sampler_matches_oracle(gpu, ops, rows, vocab):
+    """Greedy sampler: same token ids as argmax(softmax(logits / T)); ties resolve to the first index."""
+    hip, ref = ops("sampler_forward")
+    g = torch.Generator().manual_seed(rows + vocab)
+    pad = (vocab + 7) // 8 * 8
+    buf = (torch.randn((rows, pad), generator=g) * 3).to(torch.bfloat16)
+    logits = buf[:, :vocab]
+    logits[0, 5] = 50.0
+    logits[0, 3] = 50.0                      # a tie for the maximum: index 3 must win
+    if rows > 1:
+        logits[1, vocab - 1] = 60.0          # maximum in the last column
+    temps = torch.rand(rows, generator=g) + 0.1
+    want = ref(logits, temps)
+    got = hip(buf.to(gpu)[:, :vocab], temps.to(gpu))
+    assert got.dtype == torch.int64 and got.shape == (rows,)
+    assert torch.equal(got.cpu(), want)
+    assert int(got[0]) == 3

@@ -140,3 +140,65 @@ def test_decode_full_size_properties(gpu, ops, hq, hkv, lo, hi, bsz):
     sub = {"q": d["q"][pick], "k_cache": d["k_cache"], "v_cache": d["v_cache"], "cache_seqlens": d["cache_seqlens"][pick],
            "block_table": d["block_table"][pick], "scale": d["scale"]}
     assert_attention_close(got[pick], _ref(ref, sub), "sampled sequences of the full-size batch")
+
+
+@pytest.mark.parametrize("ctx,hq,hkv", [([300, 900, 31], 8, 4), ([700, 5], 4, 2), ([513, 1025], 16, 1), ([2000], 12, 6)])
+def test_decode_other_head_counts(gpu, ops, ctx, hq, hkv):
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs(ctx, hq=hq, hkv=hkv, seed=sum(ctx) + hkv, poison_tail=True)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), f"decode {hq}:{hkv}")
+
+
+def test_decode_many_short_sequences_uses_the_large_batch_plan(gpu, ops):
+    """More sequences than the plan kernel keeps in LDS (4096): prefix sums are searched in global memory;
+    a quarter of the rows are empty."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    g = torch.Generator().manual_seed(3)
+    ctx = torch.randint(0, 80, (5000,), generator=g)
+    ctx[ctx < 20] = 0
+    lens = [int(x) for x in ctx]
+    d = W.decode_inputs([max(l, 1) for l in lens], hq=4, hkv=2, seed=3)
+    d["cache_seqlens"] = torch.tensor(lens, dtype=torch.int32)
+    got = _run(hip, d, gpu).cpu()
+    want = _ref(ref, d)
+    assert (got[ctx == 0].float() == 0).all()
+    assert_attention_close(got, want, "5000 short sequences")
+
+
+@pytest.mark.parametrize("block_size", [64, 512])
+def test_decode_other_block_sizes(gpu, ops, block_size):
+    """The kernels only need the block size to be a multiple of 32; the reference uses multiples of 256."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs([1000, 300, 64], seed=block_size)
+    # re-block the same tokens: [nblk, 256, h, d] -> [nblk * 256 / bs, bs, h, d] with the table expanded / merged
+    nblk = d["k_cache"].shape[0]
+    if block_size < 256:
+        f = 256 // block_size
+        kc = d["k_cache"].view(nblk * f, block_size, 8, 128)
+        vc = d["v_cache"].view(nblk * f, block_size, 8, 128)
+        t = d["block_table"]
+        tbl = torch.where(t.unsqueeze(-1) >= 0, t.unsqueeze(-1) * f + torch.arange(f, dtype=torch.int32), torch.full((1,), -1, dtype=torch.int32))
+        tbl = tbl.reshape(t.shape[0], -1).contiguous()
+        g = {"q": d["q"].to(gpu), "k": kc.to(gpu), "v": vc.to(gpu), "t": tbl.to(gpu)}
+        got = hip(g["q"], g["k"], g["v"], cache_seqlens=d["cache_seqlens"].to(gpu), block_table=g["t"], softmax_scale=d["scale"], causal=True)
+        assert_attention_close(got, _ref(ref, d), f"block size {block_size}")
+    else:
+        d2 = W.decode_inputs([1000, 300, 64], seed=block_size)
+        # build a 512-token-block cache by pairing up 256-token blocks of a fresh layout
+        from nano_vllm_ninetoothed_amd import workloads as W2
+        lens = d2["ctx_lens"]
+        bps = [(l + 511) // 512 for l in lens]
+        nb = sum(bps)
+        gen = torch.Generator().manual_seed(9)
+        kc = torch.randn((nb, 512, 8, 128), generator=gen).to(torch.bfloat16)
+        vc = torch.randn((nb, 512, 8, 128), generator=gen).to(torch.bfloat16)
+        tbl = torch.full((3, max(bps)), -1, dtype=torch.int32)
+        perm = torch.randperm(nb, generator=gen).to(torch.int32)
+        pos = 0
+        for b, n in enumerate(bps):
+            tbl[b, :n] = perm[pos:pos + n]
+            pos += n
+        want = ref(d2["q"], kc, vc, cache_seqlens=d2["cache_seqlens"], block_table=tbl, softmax_scale=d2["scale"], causal=True)
+        got = hip(d2["q"].to(gpu), kc.to(gpu), vc.to(gpu), cache_seqlens=d2["cache_seqlens"].to(gpu), block_table=tbl.to(gpu),
+                  softmax_scale=d2["scale"], causal=True)
+        assert_attention_close(got, want, "block size 512")
