@@ -8,23 +8,33 @@
 //   is decoded so that id % 8 — the XCD a workgroup lands on — is the kv head: each XCD's L2 then only
 //   ever holds one kv head's K/V.
 //
-// Per 64-token K/V tile (double-buffered in LDS, one workgroup barrier per tile, next tile in flight from
-// HBM into registers)
-//   S^T = K . Q^T                      16 x v_mfma_f32_32x32x16_bf16 per wave; Q^T stays in registers as
-//                                      the B operand; the K operand reads run four MFMAs ahead of use
-//   softmax down the token axis:       each lane owns one q row, so max/sum are register-local plus one
-//                                      half-wave swap (v_permlane32_swap); the scale is folded into the
-//                                      exponent, the causal mask is applied on a wave's last tile only
-//   O^T += V^T . P^T                   16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
+// Per 64-token K/V tile (double-buffered in LDS, one workgroup barrier per tile), hand scheduled: every
+// MFMA opens a slot, and what the wave issues while that MFMA runs is fixed by scheduling fences
+//   block A   S^T = K . Q^T           16 x v_mfma_f32_32x32x16_bf16 per wave; Q^T stays in registers as
+//                                      the B operand; the K operand reads run four MFMAs ahead of use;
+//                                      the eight global loads of the next tile ride in the slots
+//   block B   softmax head             each lane owns one q row, so the row max is register-local
+//                                      (v_max3) plus one half-wave swap (v_permlane32_swap); rescale
+//                                      factor; the scale is folded into the exponent; the causal mask
+//                                      is applied only on tiles that reach past the wave's first row
+//   block C   O^T += V^T . P^T         16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
 //                                      already the B-operand layout, V^T comes out of LDS through
-//                                      ds_read_b64_tr_b16, also issued ahead of the MFMAs that use it
+//                                      ds_read_b64_tr_b16 four MFMAs ahead; the exponentials of the
+//                                      next 16-token block and the eight LDS stores of the next tile
+//                                      ride in the slots
 //
-// What bounds this shape: on this part ds_read_b128 streams ~210 B/clk per CU, but the transposing read
-// ds_read_b64_tr_b16 only ~65 B/clk and ds_write_b128 ~73 B/clk (measured).  With 32 query rows per wave
-// every 32-cycle MFMA of the second product needs 1 KiB of V^T through the transposing read, so the
-// LDS pipe, not the matrix pipe, sets the pace (~58 % MFMA at best).  A wave owning 64 rows halves that
-// traffic but needs ~400 VGPRs, i.e. one wave per SIMD, and then only pays off with the two products
-// and the softmax software-pipelined across tiles inside the wave.
+// What was measured on this part and shaped the kernel:
+//   * A wave issues a VALU instruction only every ~5 cycles; two waves of a SIMD together get ~2.8
+//     cycles per instruction.  MFMA and VALU work of the same or of another wave overlap only in part.
+//   * Issued in one burst after the barrier, the eight 1-KiB global loads of a wave took ~200 cycles
+//     each to issue (all eight waves of the CU queue on the same address path) and the eight LDS stores
+//     ~60 cycles each; spread over the MFMA slots both costs vanish behind the matrix pipe.
+//   * Phase-shifting the two waves of a SIMD (one in its matrix phase while the other does its softmax)
+//     was slower: the softmax then runs at the single-wave VALU issue rate.  Software-pipelining the two
+//     products across half tiles inside a wave was slower too (register pressure, two barriers per tile).
+//   * The transposing read ds_read_b64_tr_b16 delivers ~65 B/clk per CU against ~210 B/clk for
+//     ds_read_b128, but replacing it by plain reads of a pre-transposed tile did not change the run
+//     time: the LDS pipe is not what bounds this shape.
 //
 // LDS rows are padded instead of swizzled (K rows 272 B apart, V rows 320 B apart): the K operand read
 // (16 consecutive rows, one 16-byte piece) and the transposing V read (4 rows x 4 pieces) each cover
@@ -67,6 +77,14 @@ __device__ __forceinline__ float half_swap_sum(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// workgroup barrier that makes this wave's LDS traffic visible but leaves global loads in flight
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPKTile + 2 * kPVTile];  // K[2] then V[2]
@@ -169,31 +187,32 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 #pragma unroll
     for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds_v + buf * kPVTile + st_v + 16 * i * kPVStride) = r[i];
   };
-  // S^T = K . Q^T for one 64-token tile resident in LDS; lane (n, jj) reads row 32*tt + n, piece 2*kb + jj
-  const int rd_k = n * kPKStride + (jj << 4);
-  auto qk_tile = [&](int buf, f32x16 (&s)[2]) {
-    const unsigned char* kt = lds_k + buf * kPKTile + rd_k;
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
-#pragma unroll
-    for (int kb = 0; kb < 8; ++kb)
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const u32x4 w = *reinterpret_cast<const u32x4*>(kt + tt * 32 * kPKStride + kb * 32);
-        s[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), qb[kb], s[tt], 0, 0, 0);
-      }
-    // issue order: four operand reads up front, then one read per MFMA, so LDS latency hides behind
-    // the matrix pipe instead of in front of every MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  // wave-uniform base address of a tile's first token; true when the whole tile can be loaded unconditionally
+  auto tile_base = [&](const uint16_t* packed, int64_t ts, int tile, const char*& base) -> bool {
+    bool tile_ok = true;
+    if (paged) {
+      const int t0 = tile * kPBN;
+      const int blk = table[t0 / p.block_size];
+      tile_ok = blk >= 0 && blk < p.num_blocks;
+      base = reinterpret_cast<const char*>(packed + ((int64_t)(tile_ok ? blk : 0) * p.block_size + (t0 % p.block_size)) * tok_elems);
+    } else {
+      base = reinterpret_cast<const char*>(packed + (int64_t)(kbegin + tile * kPBN) * ts);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    return tile_ok && (tile + 1) * kPBN <= kv_len;
   };
+  unsigned mv_koff[4], mv_voff[4];   // this thread's byte offsets of its four pieces from a tile's base
+  {
+    const int64_t kts = paged ? tok_elems : p.k_ts, vts = paged ? tok_elems : p.v_ts;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      mv_koff[i] = (unsigned)(((int64_t)(ld_row + 16 * i) * kts + col) * 2);
+      mv_voff[i] = (unsigned)(((int64_t)(ld_row + 16 * i) * vts + col) * 2);
+    }
+  }
+  const int rd_k = n * kPKStride + (jj << 4);
+  // transposing V read: 16-lane group (d half, jj); lane addresses token row src_row of a 4-row set and
+  // the 4-wide d chunk src_chunk of the group's 16-wide window
+  const int rd_v = (4 * jj + ((lane & 15) >> 2)) * kPVStride + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3);
 
   f32x16 acc[4];
 #pragma unroll
@@ -202,14 +221,43 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
   float m_run = -INFINITY;  // running max of the raw scores of row my_row
   float l_run = 0.f;        // this lane's share of the running sum
+  u32x4 kreg[4], vreg[4];
 
-  // transposing V read: 16-lane group (d half, jj); lane addresses token row src_row of a 4-row set and
-  // the 4-wide d chunk src_chunk of the group's 16-wide window
-  const int rd_v = (4 * jj + ((lane & 15) >> 2)) * kPVStride + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3);
-
-  // online softmax of one tile's scores (already in s) and O^T += V^T . P^T
-  auto softmax_pv = [&](f32x16 (&s)[2], int buf, int j0, auto masked) {
+  // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
+  // scheduling fence are what the wave issues while that MFMA runs.
+  //   block A: S^T = K . Q^T, the eight global loads of the next tile ride in its slots
+  //   block B: row max, rescale factor, the first eight exponentials
+  //   block C: O^T += V^T . P^T, the remaining exponentials and the eight LDS stores of the next tile ride in its slots
+  auto tile_compute = [&](int tile, const char* kbase, const char* vbase, auto move, auto masked) {
+    const int buf = tile & 1;
+    f32x16 s[2];
+    {
+      const unsigned char* kt = lds_k + buf * kPKTile + rd_k;
+      u32x4 ka[16];
+      auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + (i & 1) * 32 * kPKStride + (i >> 1) * 32); };
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
+      rd(0); rd(1); rd(2); rd(3);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i >> 1], s[i & 1], 0, 0, 0);
+        if (i + 4 < 16) rd(i + 4);
+        if (decltype(move)::value && (i & 1)) {
+          const int j = i >> 1;
+          if (j < 4) kreg[j] = load16(reinterpret_cast<const uint16_t*>(kbase + mv_koff[j]));
+          else vreg[j - 4] = load16(reinterpret_cast<const uint16_t*>(vbase + mv_voff[j - 4]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    // block B
     if (decltype(masked)::value) {
+      const int j0 = tile * kPBN;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
@@ -218,78 +266,105 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
           s[tt][r] = key <= my_row + shift ? s[tt][r] : -INFINITY;
         }
     }
-    float m_loc = fmaxf(s[0][0], s[1][0]);
+    float ma = max3(s[0][0], s[0][1], s[0][2]);
+    float mb = max3(s[1][0], s[1][1], s[1][2]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) m_loc = fmaxf(m_loc, fmaxf(s[0][r], s[1][r]));
-    m_loc = half_swap_max(m_loc);
+    for (int r = 3; r < 15; r += 2) {
+      ma = max3(ma, s[0][r], s[0][r + 1]);
+      mb = max3(mb, s[1][r], s[1][r + 1]);
+    }
+    const float m_loc = half_swap_max(max3(ma, mb, fmaxf(s[0][15], s[1][15])));
     const float m_new = fmaxf(m_run, m_loc);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float mc = m_safe * p.scale_log2;
     const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - mc);
-    float psum = 0.f;
-    u32x4 pw[4];  // P^T as B operand for the four 16-token k blocks
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r], p.scale_log2, -mc));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc));
-        psum += p0 + p1;
-        pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(p0, p1);
-      }
-    l_run = l_run * alpha + psum;
     m_run = m_new;
     if (__any(alpha != 1.0f)) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
     }
-    const unsigned char* vt = lds_v + buf * kPVTile + rd_v;
+    u32x4 pw[4];   // P^T as B operand for the four 16-token k blocks
+    float ps0 = 0.f, ps1 = 0.f;
+    auto exps = [&](int q) {   // q = 0..15: elements 2q, 2q+1 of the 32 scores of this lane
+      const int tt = q >> 3, r = 2 * (q & 7);
+      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r], p.scale_log2, -mc));
+      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc));
+      if (q & 1) ps1 += e0 + e1; else ps0 += e0 + e1;
+      pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(e0, e1);
+    };
+    exps(0); exps(1); exps(2); exps(3);
+    // block C
+    {
+      const unsigned char* vt = lds_v + buf * kPVTile + rd_v;
+      unsigned char* kdst = lds_k + (buf ^ 1) * kPKTile + st_k;
+      unsigned char* vdst = lds_v + (buf ^ 1) * kPVTile + st_v;
+      s16x4 vlo[16], vhi[16];
+      auto rd = [&](int i) {
+        const int kb2 = i >> 2, dt = i & 3;
+        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + 16 * kb2 * kPVStride + 64 * dt));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + (16 * kb2 + 8) * kPVStride + 64 * dt));
+      };
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      rd(0); rd(1); rd(2); rd(3);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int kb2 = 0; kb2 < 4; ++kb2) {
-      const bf16x8 pb = __builtin_bit_cast(bf16x8, pw[kb2]);
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        // token rows 16*kb2 + 4*jj + src_row (+8 for the upper four), d = 32*dt + 16*half + 4*chunk ..
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)(vt + 16 * kb2 * kPVStride + 64 * dt));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)(vt + (16 * kb2 + 8) * kPVStride + 64 * dt));
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        const s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), pb, acc[dt], 0, 0, 0);
+      for (int i = 0; i < 16; ++i) {
+        const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
+        if (i + 4 < 16) rd(i + 4);
+        if (i < 12) exps(4 + i);
+        if (decltype(move)::value && i >= 8) {
+          const int j = i - 8;
+          if (j < 4) *reinterpret_cast<u32x4*>(kdst + 16 * j * kPKStride) = kreg[j];
+          else *reinterpret_cast<u32x4*>(vdst + 16 * (j - 4) * kPVStride) = vreg[j - 4];
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // issue order: the transposing reads of four MFMAs up front, then two reads per MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    __builtin_amdgcn_s_setprio(0);
+    l_run = l_run * alpha + (ps0 + ps1);
   };
 
-  // ---- tile loop: tile i+1 is in flight into registers while tile i is consumed out of LDS
-  u32x4 kreg[4], vreg[4];
+  // ---- tile loop.  The next tile travels HBM -> registers during block A and registers -> the other LDS
+  //      buffer during block C; that buffer was last read before this tile's barrier.
   load_tile(kptr, p.k, p.k_ts, 0, kreg);
   load_tile(vptr, p.v, p.v_ts, 0, vreg);
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
-  f32x16 s[2];
+  if (ntiles > 0) {
+    store_k(0, kreg);
+    store_v(0, vreg);
+  }
   for (int tile = 0; tile < ntiles; ++tile) {
-    const int buf = tile & 1;
-    store_k(buf, kreg);
-    store_v(buf, vreg);
-    __syncthreads();   // tile visible to all waves; the other buffer (tile-1) is free once everyone is here
-    if (tile + 1 < ntiles) {
-      load_tile(kptr, p.k, p.k_ts, tile + 1, kreg);
-      load_tile(vptr, p.v, p.v_ts, tile + 1, vreg);
+    lds_barrier();
+    const bool have_next = tile + 1 < ntiles;
+    const char* kbase = nullptr;
+    const char* vbase = nullptr;
+    bool sliced = false;
+    if (have_next && tile < my_tiles) {
+      const bool k_whole = tile_base(p.k, p.k_ts, tile + 1, kbase);
+      const bool v_whole = tile_base(p.v, p.v_ts, tile + 1, vbase);
+      sliced = k_whole && v_whole;
     }
-    if (tile < my_tiles) {
-      qk_tile(buf, s);
-      // the mask is only needed where the tile holds a key beyond the first row's horizon
-      if (tile * kPBN + kPBN - 1 > wave_row0 + shift) softmax_pv(s, buf, tile * kPBN, std::true_type{});
-      else softmax_pv(s, buf, tile * kPBN, std::false_type{});
+    // the mask is only needed where the tile holds a key beyond the first row's horizon
+    const bool masked = tile * kPBN + kPBN - 1 > wave_row0 + shift;
+    if (sliced) {
+      if (masked) tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{});
+      else tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{});
+    } else {
+      if (have_next) {
+        load_tile(kptr, p.k, p.k_ts, tile + 1, kreg);
+        load_tile(vptr, p.v, p.v_ts, tile + 1, vreg);
+      }
+      if (tile < my_tiles) {
+        if (masked) tile_compute(tile, kbase, vbase, std::false_type{}, std::true_type{});
+        else tile_compute(tile, kbase, vbase, std::false_type{}, std::false_type{});
+      }
+      if (have_next) {
+        store_k((tile + 1) & 1, kreg);
+        store_v((tile + 1) & 1, vreg);
+      }
     }
   }
 
