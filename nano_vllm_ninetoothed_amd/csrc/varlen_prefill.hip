@@ -40,6 +40,7 @@
 // (16 consecutive rows, one 16-byte piece) and the transposing V read (4 rows x 4 pieces) each cover
 // all 64 banks once, and every address a lane needs is one base register plus an immediate.
 #include "mops_common.h"
+#include <algorithm>
 #include <type_traits>
 
 namespace mops {
@@ -52,6 +53,7 @@ constexpr int kPKStride = 272;      // bytes between K rows in LDS
 constexpr int kPVStride = 320;      // bytes between V rows in LDS
 constexpr int kPKTile = kPBN * kPKStride;   // 17408
 constexpr int kPVTile = kPBN * kPVStride;   // 20480
+constexpr int kPCompactChunks = 4;  // the compact launch handles up to 64 * 4 sequences
 
 struct PrefillParams {
   const uint16_t* q;
@@ -65,6 +67,7 @@ struct PrefillParams {
   int64_t block_table_row_stride;
   int block_size, num_blocks, max_blocks_per_seq;
   int batch, total_tokens, total_k_tokens, m_tiles, hq, hkv, group;
+  int compact;   // workgroup ids enumerate only existing (q tile, sequence) pairs
   float scale_log2;
 };
 
@@ -103,16 +106,88 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     h = idx % p.hq;
     rest = idx / p.hq;
   }
-  const int b = rest % p.batch;
-  const int m = p.m_tiles - 1 - rest / p.batch;
-  const int seq_begin = p.cu_seqlens[b];
-  const int seq_len = min(p.cu_seqlens[b + 1], p.total_tokens) - seq_begin;   // query rows of this sequence
+  int b, m;
+  int seq_begin, seq_end, kbegin, kend;   // cu_seqlens_q[b], [b+1], cu_seqlens_k[b], [b+1]
+  if (p.compact) {
+    // `rest` is the rank of this workgroup's (q tile, sequence) pair in the order "highest q tile first,
+    // then sequence", counting only pairs that exist: the launch holds no workgroups for tiles past a
+    // sequence's end, so the dispatcher never idles on them.  Every wave derives the pair on its own
+    // from the tile counts of the sequences (lane l holds sequences l, l + 64, ..).
+    // One vector load per array brings every sequence's offsets into the lanes, so the chosen
+    // sequence's offsets come out of registers afterwards and not from a second trip to memory.
+    const int ln = threadIdx.x & 63;
+    int cnt[kPCompactChunks], qs[kPCompactChunks], qe[kPCompactChunks], ks[kPCompactChunks], ke[kPCompactChunks];
+#pragma unroll
+    for (int j = 0; j < kPCompactChunks; ++j) {
+      const int bb = ln + 64 * j;
+      qs[j] = qe[j] = ks[j] = ke[j] = 0;
+      if (bb < p.batch) {
+        qs[j] = p.cu_seqlens[bb];
+        qe[j] = p.cu_seqlens[bb + 1];
+        ks[j] = p.cu_seqlens_k[bb];
+        ke[j] = p.cu_seqlens_k[bb + 1];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kPCompactChunks; ++j) {
+      const int len = min(qe[j], p.total_tokens) - qs[j];
+      cnt[j] = (qs[j] >= 0 && len > 0) ? min((len + kPBM - 1) / kPBM, p.m_tiles) : 0;
+    }
+    // wave-wide sum of small non-negative integers, one ballot per bit (no trip through LDS)
+    const int sum_bits = 32 - __builtin_clz((unsigned)(kPCompactChunks * p.m_tiles));
+    auto pairs_from = [&](int mm) {   // pairs whose q tile index is >= mm
+      int c = 0;
+#pragma unroll
+      for (int j = 0; j < kPCompactChunks; ++j) c += max(0, cnt[j] - mm);
+      int total = 0;
+      for (int bit = 0; bit < sum_bits; ++bit) total += __popcll(__ballot((c >> bit) & 1)) << bit;
+      return total;
+    };
+    if (rest >= pairs_from(0)) return;
+    int lo = 0, hi = p.m_tiles - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (pairs_from(mid) > rest) lo = mid; else hi = mid - 1;
+    }
+    m = lo;
+    int r = rest - pairs_from(m + 1);   // rank among the sequences that have tile m
+    b = -1;
+    seq_begin = seq_end = kbegin = kend = 0;
+#pragma unroll
+    for (int j = 0; j < kPCompactChunks; ++j) {
+      const bool has = cnt[j] > m;
+      const unsigned long long mask = __ballot(has);
+      const int c = __popcll(mask);
+      if (b < 0) {
+        if (r < c) {
+          const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+          const unsigned long long hit = __ballot(has && before == r);
+          const int src = __builtin_ctzll(hit);
+          b = 64 * j + src;
+          seq_begin = __builtin_amdgcn_readlane(qs[j], src);
+          seq_end = __builtin_amdgcn_readlane(qe[j], src);
+          kbegin = __builtin_amdgcn_readlane(ks[j], src);
+          kend = __builtin_amdgcn_readlane(ke[j], src);
+        } else {
+          r -= c;
+        }
+      }
+    }
+    if (b < 0) return;
+  } else {
+    b = rest % p.batch;
+    m = p.m_tiles - 1 - rest / p.batch;
+    seq_begin = p.cu_seqlens[b];
+    seq_end = p.cu_seqlens[b + 1];
+    kbegin = p.cu_seqlens_k[b];
+    kend = p.cu_seqlens_k[b + 1];
+  }
+  const int seq_len = min(seq_end, p.total_tokens) - seq_begin;   // query rows of this sequence
   const int q0 = m * kPBM;
   if (seq_begin < 0 || q0 >= seq_len) return;
   // keys of this sequence: kv_len >= seq_len when a cached prefix precedes the new tokens; query row i
   // then sees keys 0 .. i + shift (bottom-right aligned causal mask)
-  const int kbegin = p.cu_seqlens_k[b];
-  int kv_len = p.cu_seqlens_k[b + 1] - kbegin;
+  int kv_len = kend - kbegin;
   const bool paged = p.block_table != nullptr;
   kv_len = max(0, min(kv_len, paged ? p.max_blocks_per_seq * p.block_size : p.total_k_tokens - kbegin));
   const int shift = kv_len - seq_len;
@@ -445,7 +520,15 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   p.hkv = (int)hkv;
   p.group = (int)(hq / hkv);
   p.scale_log2 = softmax_scale * 1.44269504088896340736f;
-  const int64_t grid = (int64_t)p.m_tiles * batch * hq;
+  // Every sequence has ceil(len / 128) q tiles, at most total_tokens / 128 + batch in all.  When that is
+  // clearly fewer than the m_tiles x batch rectangle (ragged lengths) and there are at most 256
+  // sequences, the kernel maps workgroup ids onto the existing tiles only; the mapping costs each
+  // workgroup one more trip to memory, so equal-length batches keep the rectangle.
+  int64_t pairs = (int64_t)p.m_tiles * batch;
+  const int64_t pairs_bound = total_tokens / kPBM + batch;
+  p.compact = batch <= 64 * kPCompactChunks && pairs_bound * 10 < pairs * 9;
+  if (p.compact) pairs = pairs_bound;
+  const int64_t grid = pairs * hq;
   if (grid > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
   hipLaunchKernelGGL(varlen_prefill_kernel, dim3((unsigned)grid), dim3(kPThreads), 0, (hipStream_t)stream, p);
   return finish_launch();

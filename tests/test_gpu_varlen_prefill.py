@@ -35,6 +35,20 @@ def test_prefill_matches_oracle(gpu, ops, lens, hq, hkv):
     assert_attention_close(got, _ref(ref, d), f"prefill lens={lens} {hq}:{hkv}")
 
 
+@pytest.mark.parametrize("nseq", [70, 200, 300])
+def test_prefill_many_ragged_sequences(gpu, ops, nseq):
+    """Ragged batches launch workgroups for existing q tiles only (up to 256 sequences; sequence index found
+    inside the kernel from per-lane tile counts, one 64-sequence chunk per register), larger batches use the
+    plain tile x sequence rectangle.  Lengths include empty sequences and one long straggler."""
+    hip, ref = ops("flash_attn_varlen_func")
+    gen = torch.Generator().manual_seed(nseq)
+    lens = torch.randint(0, 260, (nseq,), generator=gen).tolist()
+    lens[nseq // 2] = 700
+    lens[3] = 0
+    d = W.prefill_inputs(lens, seed=nseq)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), f"prefill {nseq} ragged sequences")
+
+
 def test_prefill_v_is_strided_view_and_max_seqlen_is_only_a_bound(gpu, ops):
     """q, k, v as nanovllm hands them: slices of one [T, 4096] qkv buffer (row stride 4096)."""
     hip, ref = ops("flash_attn_varlen_func")
