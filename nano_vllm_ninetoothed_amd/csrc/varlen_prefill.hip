@@ -341,33 +341,54 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
           s[tt][r] = key <= my_row + shift ? s[tt][r] : -INFINITY;
         }
     }
-    float ma = max3(s[0][0], s[0][1], s[0][2]);
-    float mb = max3(s[1][0], s[1][1], s[1][2]);
+    // A wave issues in order and a dependent VALU instruction waits ~20 cycles for its operand, so the
+    // softmax is written for instruction-level parallelism: four max chains, and the exponent pipeline
+    // F (scale and subtract) -> E (exp2) -> P (row sum, bf16 pack) is skewed by one MFMA slot per stage,
+    // so nothing issued in a slot depends on anything else issued in it.
+    float mx[4];
 #pragma unroll
-    for (int r = 3; r < 15; r += 2) {
-      ma = max3(ma, s[0][r], s[0][r + 1]);
-      mb = max3(mb, s[1][r], s[1][r + 1]);
-    }
-    const float m_loc = half_swap_max(max3(ma, mb, fmaxf(s[0][15], s[1][15])));
+    for (int c = 0; c < 4; ++c) mx[c] = max3(s[c >> 1][8 * (c & 1)], s[c >> 1][8 * (c & 1) + 1], s[c >> 1][8 * (c & 1) + 2]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) mx[c] = max3(mx[c], s[c >> 1][8 * (c & 1) + 3], s[c >> 1][8 * (c & 1) + 4]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) mx[c] = max3(mx[c], s[c >> 1][8 * (c & 1) + 5], s[c >> 1][8 * (c & 1) + 6]);
+    const float m01 = max3(mx[0], mx[1], s[0][7]), m23 = max3(mx[2], mx[3], s[0][15]);
+    const float m_loc = half_swap_max(max3(m01, m23, fmaxf(s[1][7], s[1][15])));
     const float m_new = fmaxf(m_run, m_loc);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float mc = m_safe * p.scale_log2;
     const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - mc);
     m_run = m_new;
+    u32x4 pw[4];   // P^T as B operand for the four 16-token k blocks
+    float ps0 = 0.f, ps1 = 0.f;
+    float f0[16], f1[16];   // per element pair q = 0..15 (elements 2q, 2q+1 of this lane's 32 scores): stage values
+    auto stage_f = [&](int q) {
+      const int tt = q >> 3, r = 2 * (q & 7);
+      f0[q] = __builtin_fmaf(s[tt][r], p.scale_log2, -mc);
+      f1[q] = __builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc);
+    };
+    auto stage_e = [&](int q) {
+      f0[q] = __builtin_amdgcn_exp2f(f0[q]);
+      f1[q] = __builtin_amdgcn_exp2f(f1[q]);
+    };
+    auto stage_p = [&](int q) {
+      const int tt = q >> 3, r = 2 * (q & 7);
+      if (q & 1) ps1 += f0[q] + f1[q]; else ps0 += f0[q] + f1[q];
+      pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(f0[q], f1[q]);
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < 6; ++q) stage_f(q);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < 5; ++q) stage_e(q);
+    __builtin_amdgcn_sched_barrier(0);
     if (__any(alpha != 1.0f)) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
     }
-    u32x4 pw[4];   // P^T as B operand for the four 16-token k blocks
-    float ps0 = 0.f, ps1 = 0.f;
-    auto exps = [&](int q) {   // q = 0..15: elements 2q, 2q+1 of the 32 scores of this lane
-      const int tt = q >> 3, r = 2 * (q & 7);
-      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r], p.scale_log2, -mc));
-      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc));
-      if (q & 1) ps1 += e0 + e1; else ps0 += e0 + e1;
-      pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(e0, e1);
-    };
-    exps(0); exps(1); exps(2); exps(3);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_p(q);
     // block C
     {
       const unsigned char* vt = lds_v + buf * kPVTile + rd_v;
@@ -388,7 +409,10 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
         acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
         if (i + 4 < 16) rd(i + 4);
-        if (i < 12) exps(4 + i);
+        // slot i finishes pair i + 4 (needed from slot 4 * ((i + 4) / 4) on), exponentiates i + 5, scales i + 6
+        if (i + 4 < 16) stage_p(i + 4);
+        if (i + 5 < 16) stage_e(i + 5);
+        if (i + 6 < 16) stage_f(i + 6);
         if (decltype(move)::value && i >= 8) {
           const int j = i - 8;
           if (j < 4) *reinterpret_cast<u32x4*>(kdst + 16 * j * kPKStride) = kreg[j];
@@ -411,7 +435,25 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     store_k(0, kreg);
     store_v(0, vreg);
   }
-  for (int tile = 0; tile < ntiles; ++tile) {
+  // Steady prefix of the loop: tiles this wave computes without a mask and whose successor is a whole
+  // tile of a packed K/V.  There the per-tile bookkeeping is two pointer increments; everything else
+  // (paged caches, partial tiles, the diagonal, tiles this wave skips) takes the general loop below.
+  // Both loops hold exactly one barrier per tile, so the waves of a workgroup may sit in different ones.
+  int tile = 0;
+  if (!paged) {
+    const int unmasked = wave_row0 + shift + 1 >= 0 ? (wave_row0 + shift + 1) / kPBN : 0;
+    const int n_fast = min(min(unmasked, my_tiles), min(kv_len / kPBN - 1, ntiles - 1));
+    const char* kbase = reinterpret_cast<const char*>(p.k + (int64_t)(kbegin + kPBN) * p.k_ts);
+    const char* vbase = reinterpret_cast<const char*>(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
+    const int64_t kstep = (int64_t)kPBN * p.k_ts * 2, vstep = (int64_t)kPBN * p.v_ts * 2;
+    for (; tile < n_fast; ++tile) {
+      lds_barrier();
+      tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{});
+      kbase += kstep;
+      vbase += vstep;
+    }
+  }
+  for (; tile < ntiles; ++tile) {
     lds_barrier();
     const bool have_next = tile + 1 < ntiles;
     const char* kbase = nullptr;
