@@ -81,11 +81,10 @@ __device__ __forceinline__ float half_swap_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
+// max of three; the compiler fuses the nested form into one v_max3_f32.  It has to stay a compiler-visible
+// operation: the wait states between an MFMA and the first VALU read of its result are inserted by the
+// compiler's hazard recognizer, which does not look inside inline assembly.
+__device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 // workgroup barrier that makes this wave's LDS traffic visible but leaves global loads in flight
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -435,20 +434,21 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     store_k(0, kreg);
     store_v(0, vreg);
   }
-  // Steady prefix of the loop: tiles this wave computes without a mask and whose successor is a whole
-  // tile of a packed K/V.  There the per-tile bookkeeping is two pointer increments; everything else
-  // (paged caches, partial tiles, the diagonal, tiles this wave skips) takes the general loop below.
-  // Both loops hold exactly one barrier per tile, so the waves of a workgroup may sit in different ones.
+  // Steady prefix of the loop: tiles this wave computes and whose successor is a whole tile of a packed
+  // K/V.  There the per-tile bookkeeping is two pointer increments; everything else (paged caches,
+  // partial tiles, the last tile, tiles this wave skips) takes the general loop below.  Both loops hold
+  // exactly one barrier per tile, so the waves of a workgroup may sit in different ones.
   int tile = 0;
   if (!paged) {
-    const int unmasked = wave_row0 + shift + 1 >= 0 ? (wave_row0 + shift + 1) / kPBN : 0;
-    const int n_fast = min(min(unmasked, my_tiles), min(kv_len / kPBN - 1, ntiles - 1));
+    const int n_fast = min(my_tiles, min(kv_len / kPBN - 1, ntiles - 1));
+    const int unmasked = wave_row0 + shift + 1 >= 0 ? (wave_row0 + shift + 1) / kPBN : 0;   // tiles wholly below the first row's horizon
     const char* kbase = reinterpret_cast<const char*>(p.k + (int64_t)(kbegin + kPBN) * p.k_ts);
     const char* vbase = reinterpret_cast<const char*>(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
     const int64_t kstep = (int64_t)kPBN * p.k_ts * 2, vstep = (int64_t)kPBN * p.v_ts * 2;
     for (; tile < n_fast; ++tile) {
       lds_barrier();
-      tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{});
+      if (tile < unmasked) tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{});
+      else tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{});
       kbase += kstep;
       vbase += vstep;
     }

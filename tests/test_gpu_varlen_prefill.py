@@ -127,6 +127,22 @@ def test_prefill_with_cached_prefix_matches_oracle(gpu, ops, new, prefix, hq, hk
     assert_bit_exact(got_packed, got, "packed keys with cu_seqlens_k vs paged keys")
 
 
+def test_prefill_is_bitwise_reproducible(gpu, ops):
+    """The same launch repeated gives the same bits (plain, packed-with-prefix and paged inputs).  Guards the
+    kernel's hand-placed instruction order: a VALU read of an MFMA result that comes too early returns
+    a mix of old and new register contents, which shows up as run-to-run differences of an ulp."""
+    hip, _ = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([700, 130, 1025], seed=91)
+    first = _run(hip, d, gpu).clone()
+    for _ in range(30):
+        assert_bit_exact(_run(hip, d, gpu), first, "plain prefill, repeated launch")
+    dp = W.prefix_prefill_inputs([513, 100], [1024, 256], hq=16, hkv=8, seed=92)
+    for paged in (True, False):
+        first = _run_prefix(hip, dp, gpu, paged=paged).clone()
+        for _ in range(30):
+            assert_bit_exact(_run_prefix(hip, dp, gpu, paged=paged), first, f"prefix prefill paged={paged}, repeated launch")
+
+
 def test_prefix_prefill_last_row_equals_decode(gpu, ops):
     pre, _ = ops("flash_attn_varlen_func")
     dec, _ = ops("flash_attn_with_kvcache")
