@@ -3,10 +3,10 @@
 //
 // Work decomposition
 //   workgroup (256 lanes, 4 waves) = one 128-row Q tile of one sequence for one query head; wave w owns
-//   rows 32w..32w+31.  The launch is sized from max_seqlen (tiles past a sequence's end exit at once),
-//   the tiles with the longest causal prefix are dispatched first, and with 8 kv heads the workgroup id
-//   is decoded so that id % 8 — the XCD a workgroup lands on — is the kv head: each XCD's L2 then only
-//   ever holds one kv head's K/V.
+//   rows 32w..32w+31; two workgroups per CU.  Tiles with the longest causal prefix are dispatched first,
+//   and with 8 kv heads the workgroup id is decoded so that id % 8 — the XCD a workgroup lands on — is
+//   the kv head: each XCD's L2 then only ever holds one kv head's K/V.  Ragged batches launch workgroups
+//   for existing q tiles only (the kernel maps the workgroup's rank to its tile and sequence).
 //
 // Per 64-token K/V tile (double-buffered in LDS, one workgroup barrier per tile), hand scheduled: every
 // MFMA opens a slot, and what the wave issues while that MFMA runs is fixed by scheduling fences
@@ -14,27 +14,38 @@
 //                                      the B operand; the K operand reads run four MFMAs ahead of use;
 //                                      the eight global loads of the next tile ride in the slots
 //   block B   softmax head             each lane owns one q row, so the row max is register-local
-//                                      (v_max3) plus one half-wave swap (v_permlane32_swap); rescale
-//                                      factor; the scale is folded into the exponent; the causal mask
-//                                      is applied only on tiles that reach past the wave's first row
+//                                      (four v_max3 chains) plus one half-wave swap
+//                                      (v_permlane32_swap); rescale factor; the scale is folded into
+//                                      the exponent; the causal mask is applied only on tiles that
+//                                      reach past the wave's first row
 //   block C   O^T += V^T . P^T         16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
 //                                      already the B-operand layout, V^T comes out of LDS through
-//                                      ds_read_b64_tr_b16 four MFMAs ahead; the exponentials of the
-//                                      next 16-token block and the eight LDS stores of the next tile
-//                                      ride in the slots
+//                                      ds_read_b64_tr_b16 four MFMAs ahead; the exponent pipeline
+//                                      (scale, exp2, sum and pack), skewed one slot per stage, and the
+//                                      eight LDS stores of the next tile ride in the slots
+// In the steady part of the tile loop the per-tile bookkeeping is two pointer increments.
 //
 // What was measured on this part and shaped the kernel:
-//   * A wave issues a VALU instruction only every ~5 cycles; two waves of a SIMD together get ~2.8
-//     cycles per instruction.  MFMA and VALU work of the same or of another wave overlap only in part.
+//   * A wave issues a VALU instruction every ~5 cycles (a dependent one every ~9, an exp2 every ~8);
+//     two waves of a SIMD together get ~2.8 cycles per instruction.  MFMA and VALU work of the same or
+//     of another wave overlap only in part, and a second wave per SIMD adds only ~26 % throughput to
+//     this kernel: what counts is the length of a wave's own instruction stream per tile.
+//   * Address and bounds bookkeeping between the barrier and the first MFMA took ~900 cycles per tile
+//     (a quarter of the tile) before the steady loop replaced it by pointer increments.
 //   * Issued in one burst after the barrier, the eight 1-KiB global loads of a wave took ~200 cycles
 //     each to issue (all eight waves of the CU queue on the same address path) and the eight LDS stores
 //     ~60 cycles each; spread over the MFMA slots both costs vanish behind the matrix pipe.
-//   * Phase-shifting the two waves of a SIMD (one in its matrix phase while the other does its softmax)
-//     was slower: the softmax then runs at the single-wave VALU issue rate.  Software-pipelining the two
-//     products across half tiles inside a wave was slower too (register pressure, two barriers per tile).
+//   * Every VALU read of an MFMA result goes through compiler-visible code: the wait states between an
+//     MFMA and the first read of its result are software-inserted, and an inline-assembly v_max3 on the
+//     scores read half-written registers now and then (results then differ by an ulp from run to run).
+//   * Variants that were slower on the benchmark shape: phase-shifting the two waves of a SIMD in
+//     256-row, 8-wave workgroups (one in its matrix phase while the other does its softmax; +4 % on
+//     8192-token sequences, -10 % on 128..2048-token ones), one wave per SIMD owning two 32-row slabs
+//     (512 registers; the compiler shuttles values between the two register files), software-pipelining
+//     the two products across half tiles inside a wave (register pressure, two barriers per tile).
 //   * The transposing read ds_read_b64_tr_b16 delivers ~65 B/clk per CU against ~210 B/clk for
-//     ds_read_b128, but replacing it by plain reads of a pre-transposed tile did not change the run
-//     time: the LDS pipe is not what bounds this shape.
+//     ds_read_b128, but replacing it by plain reads of a pre-transposed tile changed the run time by
+//     2 %: the LDS pipe is not what bounds this shape.
 //
 // LDS rows are padded instead of swizzled (K rows 272 B apart, V rows 320 B apart): the K operand read
 // (16 consecutive rows, one 16-byte piece) and the transposing V read (4 rows x 4 pieces) each cover
