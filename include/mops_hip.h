@@ -201,6 +201,25 @@ int mops_hip_apply_rotary_emb(const void* x, int64_t x_token_stride, int64_t x_h
 int mops_hip_sampler_argmax(const void* logits, int64_t row_stride, int64_t* out, int64_t rows, int64_t n,
                             void* stream);
 
+/*
+ * qk_norm_rope_store — the four small steps between the qkv projection and the attention call of a Qwen3
+ * layer as one launch: per-head RMSNorm of q and k, rotary embedding of both, scatter of k and v into the
+ * paged cache.  Replaces the sequence nanovllm/models/qwen3.py:74-80 (q_norm, k_norm, rotary_emb) +
+ * nanovllm/layers/attention.py:29-31 (store_kvcache), i.e. mops rms_forward x2, apply_rotary_emb x2 and
+ * store_kvcache, and is bit-identical to running those (same roundings in the same order).
+ * qkv: [tokens, (hq + 2*hkv) * 128] bf16, q heads first, then k, then v, token stride in elements (% 8 == 0);
+ * q_weight, k_weight: [128] bf16; cos, sin: fp32 [tokens, 64] with token strides; slot_mapping: int32 [tokens],
+ * -1 or out of range = skip the cache rows of that token; q_out: [tokens, hq, 128] bf16; k_out: [tokens, hkv, 128]
+ * bf16 or NULL when the rotated keys are only needed in the cache (decode); caches: [num_slots, hkv, 128] bf16.
+ * v is not copied out: the attention call reads it from qkv as a strided view.
+ */
+int mops_hip_qk_norm_rope_store(const void* qkv, int64_t qkv_token_stride, const void* q_weight,
+                                const void* k_weight, const float* cos, int64_t cos_token_stride,
+                                const float* sin, int64_t sin_token_stride,
+                                const int32_t* slot_mapping, void* q_out, void* k_out, void* k_cache,
+                                void* v_cache, int64_t tokens, int64_t hq, int64_t hkv, int64_t head_dim,
+                                int64_t num_slots, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,9 +39,12 @@ SIGNATURES = {
     "mops_hip_apply_rotary_emb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p]),
     "mops_hip_sampler_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
+    "mops_hip_qk_norm_rope_store": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+                                            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                            c_int64, c_int64, c_float, c_void_p]),
 }
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib = None
 

@@ -80,6 +80,9 @@ class Engine:
             if op is None and name != "softmax":
                 raise RuntimeError(f"backend {backend} does not provide {name}")
             setattr(self, "op_" + name, op)
+        # the fused q_norm + k_norm + rotary + store_kvcache launch, where the backend has it
+        self.op_qk_norm_rope_store = mops.get_op("qk_norm_rope_store", backend) if mops.has_op("qk_norm_rope_store", backend) else None
+        self.use_fused_qk = True
 
         g = torch.Generator(device=self.dev).manual_seed(seed)
 
@@ -158,9 +161,10 @@ class Engine:
         return self.op_linear(self.g_out[:bs], self.embed)
 
     # ------------------------------------------------------------------ model
-    def _attention(self, layer_id, q, k, v, ctx):
+    def _attention(self, layer_id, q, k, v, ctx, stored=False):
         k_cache, v_cache = self.kv_cache[0, layer_id], self.kv_cache[1, layer_id]
-        self.op_store_kvcache(k, v, k_cache, v_cache, ctx["slot_mapping"])
+        if not stored:
+            self.op_store_kvcache(k, v, k_cache, v_cache, ctx["slot_mapping"])
         if ctx["is_prefill"]:
             return self.op_flash_attn_varlen_func(q, k, v, max_seqlen_q=ctx["max_seqlen"], cu_seqlens_q=ctx["cu_seqlens"],
                                                   max_seqlen_k=ctx["max_seqlen"], cu_seqlens_k=ctx["cu_seqlens"],
@@ -180,13 +184,19 @@ class Engine:
             else:
                 h, residual = self.op_add_rms_forward(h, residual, L["input_norm"], s.rms_eps)
             qkv = self.op_linear(h, L["qkv"])
-            q, k, v = qkv.split([self.q_size, self.kv_size, self.kv_size], dim=-1)
-            q = self.op_rms_forward(q.view(-1, s.num_heads, s.head_dim), L["q_norm"], s.rms_eps)
-            k = self.op_rms_forward(k.view(-1, s.num_kv_heads, s.head_dim), L["k_norm"], s.rms_eps)
-            v = v.view(-1, s.num_kv_heads, s.head_dim)
-            q = self.op_apply_rotary_emb(q, cos, sin)
-            k = self.op_apply_rotary_emb(k, cos, sin)
-            o = self._attention(i, q, k, v, ctx)
+            if self.op_qk_norm_rope_store is not None and self.use_fused_qk:
+                q, k, v = self.op_qk_norm_rope_store(qkv, L["q_norm"], L["k_norm"], s.rms_eps, cos, sin, self.kv_cache[0, i],
+                                                     self.kv_cache[1, i], ctx["slot_mapping"], s.num_heads, s.num_kv_heads,
+                                                     need_k=ctx["is_prefill"])
+                o = self._attention(i, q, k, v, ctx, stored=True)
+            else:
+                q, k, v = qkv.split([self.q_size, self.kv_size, self.kv_size], dim=-1)
+                q = self.op_rms_forward(q.view(-1, s.num_heads, s.head_dim), L["q_norm"], s.rms_eps)
+                k = self.op_rms_forward(k.view(-1, s.num_kv_heads, s.head_dim), L["k_norm"], s.rms_eps)
+                v = v.view(-1, s.num_kv_heads, s.head_dim)
+                q = self.op_apply_rotary_emb(q, cos, sin)
+                k = self.op_apply_rotary_emb(k, cos, sin)
+                o = self._attention(i, q, k, v, ctx)
             h = self.op_linear(o.flatten(1, -1), L["o"])
             h, residual = self.op_add_rms_forward(h, residual, L["post_norm"], s.rms_eps)
             gate, up = self.op_linear(h, L["gate_up"]).chunk(2, -1)

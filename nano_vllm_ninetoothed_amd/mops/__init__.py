@@ -9,7 +9,7 @@ test harness (or the reference's own backends) can register into them and be fet
 """
 import os
 
-from .registry import get_current_backend, get_op, register_op, set_current_backend
+from .registry import get_current_backend, get_op, has_op, register_op, set_current_backend
 
 _BACKEND = os.environ.get("BACKEND", "hip").lower()
 set_current_backend(_BACKEND)
@@ -30,6 +30,9 @@ OP_NAMES = (
     "flash_attn_with_kvcache",
 )
 
+# Operators this backend adds to the reference's eleven; a backend need not provide them.
+EXTENSION_OP_NAMES = ("qk_norm_rope_store",)
+
 
 def rebind(backend: str = None) -> None:
     """(Re)binds the module-level op handles to `backend` (default: the current one)."""
@@ -38,6 +41,8 @@ def rebind(backend: str = None) -> None:
     g = globals()
     for name in OP_NAMES:
         g[name] = get_op(name)
+    for name in EXTENSION_OP_NAMES:
+        g[name] = get_op(name) if has_op(name) else None
 
 
 rebind()

@@ -318,5 +318,42 @@ def apply_rotary_emb(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> t
 
 
 @register_hip_op
+def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float,
+                       cos: torch.Tensor, sin: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                       slot_mapping: torch.Tensor, num_heads: int, num_kv_heads: int, need_k: bool = True):
+    """Extension op (not one of the reference's eleven): q_norm, k_norm, rotary embedding of q and k and
+    store_kvcache of the rotated k and of v in one launch; bit-identical to
+    rms_forward x2 -> apply_rotary_emb x2 -> store_kvcache (nanovllm/models/qwen3.py:74-80,
+    nanovllm/layers/attention.py:29-31).  qkv is the [tokens, (Hq + 2*Hkv) * 128] output of the qkv projection.
+    Returns (q [tokens, Hq, 128], k [tokens, Hkv, 128] or None when need_k is False, v as a view of qkv)."""
+    _require_cuda_bf16("qkv", qkv)
+    for name, t in (("q_weight", q_weight), ("k_weight", k_weight), ("k_cache", k_cache), ("v_cache", v_cache)):
+        _require_cuda_bf16(name, t)
+    head_dim = q_weight.numel()
+    heads = num_heads + 2 * num_kv_heads
+    _require(qkv.dim() == 2 and qkv.shape[1] == heads * head_dim and qkv.stride(1) == 1, "qkv must be [tokens, (Hq + 2*Hkv) * head_dim]")
+    _require(k_weight.numel() == head_dim and q_weight.is_contiguous() and k_weight.is_contiguous(), "norm weights must be [head_dim]")
+    t = qkv.shape[0]
+    half = head_dim // 2
+    _require(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_cuda and sin.is_cuda, "cos/sin must be fp32 GPU tensors")
+    _require(cos.shape == sin.shape and cos.numel() == t * half and cos.shape[-1] == half and cos.stride(-1) == 1
+             and sin.stride(-1) == 1, "cos/sin must be [tokens, 1, head_dim/2] with a contiguous last dim")
+    _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape and k_cache.is_contiguous() and v_cache.is_contiguous()
+             and k_cache.shape[2] == num_kv_heads and k_cache.shape[3] == head_dim, "caches must be contiguous [blocks, block_size, Hkv, head_dim]")
+    _require(slot_mapping.numel() == t and slot_mapping.dtype == torch.int32 and slot_mapping.is_cuda and slot_mapping.is_contiguous(),
+             "slot_mapping must be a contiguous int32 GPU tensor with one entry per token")
+    q = torch.empty((t, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    k = torch.empty((t, num_kv_heads, head_dim), dtype=qkv.dtype, device=qkv.device) if need_k else None
+    st = _capi.load().mops_hip_qk_norm_rope_store(
+        qkv.data_ptr(), qkv.stride(0) if t > 1 else heads * head_dim, q_weight.data_ptr(), k_weight.data_ptr(),
+        cos.data_ptr(), cos.stride(0) if t > 1 else half, sin.data_ptr(), sin.stride(0) if t > 1 else half,
+        slot_mapping.data_ptr(), q.data_ptr(), k.data_ptr() if need_k else None, k_cache.data_ptr(), v_cache.data_ptr(),
+        t, num_heads, num_kv_heads, head_dim, k_cache.shape[0] * k_cache.shape[1], float(eps), _stream(qkv))
+    _capi.check("mops_hip_qk_norm_rope_store", st)
+    v = qkv[:, (num_heads + num_kv_heads) * head_dim:].view(t, num_kv_heads, head_dim)
+    return q, k, v
+
+
+@register_hip_op
 def softmax(x: torch.Tensor, dim: int = -1):
     return torch.softmax(x, dim=dim)

@@ -39,6 +39,11 @@ def register_op(backend: str):
     return decorator
 
 
+def has_op(op_name: str, backend: str = None) -> bool:
+    """True if `backend` (default: the current one) registered `op_name`; unlike get_op it prints nothing."""
+    return op_name in _BACKEND_REGISTRY.get(backend if backend is not None else _CURRENT_BACKEND, {})
+
+
 def get_op(op_name: str, backend: str = None) -> Callable:
     if backend is None:
         backend = _CURRENT_BACKEND

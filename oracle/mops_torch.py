@@ -179,3 +179,19 @@ def sampler_forward(logits, temperatures):
 def apply_rotary_emb(x, cos, sin):
     x1, x2 = torch.chunk(x.float(), 2, dim=-1)
     return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1).to(x.dtype)
+
+
+@_fresh
+def qk_norm_rope_store(qkv, q_weight, k_weight, eps, cos, sin, k_cache, v_cache, slot_mapping, num_heads, num_kv_heads,
+                       need_k=True):
+    """The hip backend's extension op, restated as the sequence it fuses: q_norm, k_norm, rotary embedding
+    of q and k, store_kvcache (nanovllm/models/qwen3.py:74-80, nanovllm/layers/attention.py:29-31)."""
+    d = q_weight.numel()
+    q, k, v = qkv.split([num_heads * d, num_kv_heads * d, num_kv_heads * d], dim=-1)
+    q = rms_forward(q.reshape(-1, num_heads, d), q_weight, eps)
+    k = rms_forward(k.reshape(-1, num_kv_heads, d), k_weight, eps)
+    v = v.reshape(-1, num_kv_heads, d)
+    q = apply_rotary_emb(q, cos, sin)
+    k = apply_rotary_emb(k, cos, sin)
+    store_kvcache(k, v, k_cache, v_cache, slot_mapping)
+    return q, (k if need_k else None), v

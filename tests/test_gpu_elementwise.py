@@ -68,3 +68,53 @@ def test_sampler_matches_oracle(gpu, ops, rows, vocab):
     assert got.dtype == torch.int64 and got.shape == (rows,)
     assert torch.equal(got.cpu(), want)
     assert int(got[0]) == 3
+
+
+@pytest.mark.parametrize("tokens,hq,hkv,need_k", [(1, 16, 8, True), (5, 16, 8, False), (300, 16, 8, True), (64, 32, 8, False), (33, 8, 1, True)])
+def test_fused_qk_norm_rope_store_equals_the_separate_ops(gpu, tokens, hq, hkv, need_k):
+    """qk_norm_rope_store against the sequence it replaces, both through the hip backend: bit-identical q, k
+    and caches, skipped slots untouched; and against the oracle's composition within the norm criterion."""
+    import oracle.mops_torch  # noqa: F401
+    from nano_vllm_ninetoothed_amd import mops
+    d, block = 128, 256
+    g = torch.Generator().manual_seed(tokens * 7 + hq)
+    qkv = torch.randn((tokens, (hq + 2 * hkv) * d), generator=g).to(torch.bfloat16)
+    wq = (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    wk = (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+    pos = torch.randint(0, 4096, (tokens,), generator=g)
+    inv = 1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    fr = torch.outer(pos.float(), inv)
+    cos, sin = fr.cos().unsqueeze(1), fr.sin().unsqueeze(1)
+    nblocks = (tokens + block - 1) // block + 1
+    slots = torch.randperm(nblocks * block, generator=g)[:tokens].to(torch.int32)
+    if tokens > 2:
+        slots[1] = -1
+    sentinel = torch.full((nblocks, block, hkv, d), -7.0, dtype=torch.bfloat16)
+
+    def run(backend, device):
+        kc, vc = sentinel.clone().to(device), sentinel.clone().to(device)
+        args = [t.to(device) for t in (qkv, wq, wk)]
+        c, s_, sl = cos.to(device), sin.to(device), slots.to(device)
+        fused = mops.get_op("qk_norm_rope_store", backend)(args[0], args[1], args[2], 1e-6, c, s_, kc, vc, sl, hq, hkv, need_k=need_k)
+        return fused, kc, vc, (args, c, s_, sl)
+
+    (q_f, k_f, v_f), kc_f, vc_f, (a, c, s_, sl) = run("hip", gpu)
+    # the separate hip ops
+    q_in, k_in, v_in = a[0].split([hq * d, hkv * d, hkv * d], dim=-1)
+    q_s = mops.get_op("apply_rotary_emb", "hip")(mops.get_op("rms_forward", "hip")(q_in.view(-1, hq, d), a[1], 1e-6), c, s_)
+    k_s = mops.get_op("apply_rotary_emb", "hip")(mops.get_op("rms_forward", "hip")(k_in.view(-1, hkv, d), a[2], 1e-6), c, s_)
+    kc_s, vc_s = sentinel.clone().to(gpu), sentinel.clone().to(gpu)
+    mops.get_op("store_kvcache", "hip")(k_s, v_in.view(-1, hkv, d), kc_s, vc_s, sl)
+    assert_bit_exact(q_f, q_s, "fused q vs rms_forward + apply_rotary_emb")
+    if need_k:
+        assert_bit_exact(k_f, k_s, "fused k vs rms_forward + apply_rotary_emb")
+    else:
+        assert k_f is None
+    assert_bit_exact(kc_f, kc_s, "k cache after the fused op vs after store_kvcache")
+    assert_bit_exact(vc_f, vc_s, "v cache after the fused op vs after store_kvcache")
+    assert_bit_exact(v_f, v_in.view(-1, hkv, d), "v is the view of qkv")
+    # oracle composition (CPU): same values up to the norm's double rounding
+    (q_o, k_o, _), kc_o, vc_o, _ = run("torch", "cpu")
+    assert (q_f.float().cpu() - q_o.float()).abs().max() <= 0.0625
+    assert_bit_exact(vc_f, vc_o, "v cache vs oracle")
+    assert ((kc_f.float().cpu() - kc_o.float()).abs() <= 0.0625).all()

@@ -41,6 +41,33 @@ def test_prefill_and_decode_logits_match_oracle_backend(gpu):
         assert err <= 0.05 * b.abs().max().item() + 1e-3, f"{what} logits differ by {err}"
 
 
+def test_fused_qk_step_gives_the_same_logits_and_cache_as_the_separate_ops(gpu):
+    """The engine with the fused q_norm/k_norm/rotary/store launch and the same engine with the four separate
+    ops produce bit-identical prefill and decode logits and KV caches."""
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    shape = Qwen3Shape(num_layers=2, vocab=2048)
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, 2048, (n,), generator=g).tolist() for n in (129, 3, 256)]
+    res = []
+    for fused in (True, False):
+        eng = Engine(shape, backend="hip", num_blocks=24, seed=3, device=str(gpu))
+        assert eng.op_qk_norm_rope_store is not None
+        eng.use_fused_qk = fused
+        for p in prompts:
+            eng.add_request(p, 4)
+        seqs, _ = eng._schedule()
+        ids, pos, ctx = eng._prepare_prefill(seqs)
+        lp = eng.forward(ids, pos, ctx)
+        for q in seqs:
+            q.token_ids.append(11)
+        seqs2, _ = eng._schedule()
+        ids, pos, ctx = eng._prepare_decode(seqs2)
+        ld = eng.forward(ids, pos, ctx)
+        res.append((lp.cpu(), ld.cpu(), eng.kv_cache.cpu()))
+    for a, b, what in zip(res[0], res[1], ("prefill logits", "decode logits", "kv cache")):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)), what
+
+
 def test_generate_respects_max_tokens_and_frees_blocks(gpu):
     hip, _ = _engines(gpu)
     g = torch.Generator().manual_seed(1)
