@@ -65,6 +65,7 @@ struct DecodeParams {
   int batch, hq, hkv, group;       // group = hq / hkv  (<= 16)
   int block_size, num_blocks, max_blocks_per_seq;
   int ncols;
+  int min_per_col;      // shortest run of stages a column is given
   float scale_log2;                // softmax_scale * log2(e)
 };
 
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(kPlanThreads) void paged_decode_plan_kernel(const D
     p.prefix[p.batch] = total;
     if (use_lds) prefix_lds[p.batch] = total;
   }
-  const int per_col = max(1, (total + p.ncols - 1) / p.ncols);
+  const int per_col = max(p.min_per_col, (total + p.ncols - 1) / p.ncols);
   if (tid == 0) {
     p.hdr[0] = total;
     p.hdr[1] = per_col;
@@ -432,17 +433,33 @@ __global__ __launch_bounds__(kWave) void paged_decode_combine_kernel(const Decod
   if (j0 == j1) return;  // one piece: written directly by the main kernel
   // partial of column j: slot 1 in the column where the sequence begins, slot 0 in the following ones
   auto slot_of = [&](int j) -> int64_t { return ((int64_t)j * 2 + (j == j0 ? 1 : 0)) * p.hq + h; };
+  // A short batch of long sequences spreads one sequence over many columns, so neither pass may be a
+  // chain of dependent loads: the maxima are read one per lane and reduced across the wave, and the
+  // weighted sum keeps eight independent partial rows in flight.
+  const int n_parts = j1 - j0 + 1;
   float m = -INFINITY;
-  for (int j = j0; j <= j1; ++j) m = fmaxf(m, p.ws_ml[2 * slot_of(j)]);
+  for (int i = lane; i < n_parts; i += kWave) m = fmaxf(m, p.ws_ml[2 * slot_of(j0 + i)]);
+  m = group_max<kWave>(m);
   const float m_safe = (m == -INFINITY) ? 0.f : m;
   float l = 0.f, o0 = 0.f, o1 = 0.f;
-  for (int j = j0; j <= j1; ++j) {
-    const int64_t sl = slot_of(j);
-    const float w = __builtin_amdgcn_exp2f(p.ws_ml[2 * sl] - m_safe);
-    l += w * p.ws_ml[2 * sl + 1];
-    const float2 a = *reinterpret_cast<const float2*>(p.ws_acc + sl * kHeadDim + 2 * lane);
-    o0 += w * a.x;
-    o1 += w * a.y;
+  for (int i0 = 0; i0 < n_parts; i0 += 8) {
+    float ml[8][2];
+    float2 a[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const bool ok = i0 + u < n_parts;
+      const int64_t sl = slot_of(j0 + (ok ? i0 + u : 0));
+      ml[u][0] = ok ? p.ws_ml[2 * sl] : -INFINITY;
+      ml[u][1] = ok ? p.ws_ml[2 * sl + 1] : 0.f;
+      a[u] = *reinterpret_cast<const float2*>(p.ws_acc + sl * kHeadDim + 2 * lane);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {   // same order of additions as a plain loop over the columns
+      const float w = (i0 + u < n_parts) ? __builtin_amdgcn_exp2f(ml[u][0] - m_safe) : 0.f;
+      l += w * ml[u][1];
+      o0 += w * a[u].x;
+      o1 += w * a[u].y;
+    }
   }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
   reinterpret_cast<uint32_t*>(p.out + (int64_t)bh * kHeadDim)[lane] = pack_bf16x2(o0 * inv, o1 * inv);
@@ -554,6 +571,12 @@ extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_st
   p.num_blocks = (int)num_blocks;
   p.max_blocks_per_seq = (int)max_blocks_per_seq;
   p.ncols = choose_ncols(hkv);
+  {
+    // With few stages in all (a short batch) runs of one stage would spread a sequence over as many partial
+    // results as it has stages; two stages per column halve the combine's work at no cost to the streaming.
+    static const int forced = env_int("MOPS_HIP_DECODE_MIN_PER_COL");  // tuning override
+    p.min_per_col = forced > 0 ? forced : 2;
+  }
   p.scale_log2 = softmax_scale * 1.44269504088896340736f;
   const WorkspaceLayout w = workspace_layout(batch, hq, p.ncols);
   if (!workspace || workspace_bytes < w.total) return MOPS_HIP_EWORKSPACE;

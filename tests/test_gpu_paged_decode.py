@@ -41,6 +41,15 @@ def test_decode_batch_of_ragged_contexts(gpu, ops):
     assert_attention_close(_run(hip, d, gpu), _ref(ref, d), "ragged batch")
 
 
+@pytest.mark.parametrize("ctx", [[16384], [9000, 5], [70] * 3 + [12000]])
+def test_decode_short_batch_of_long_contexts(gpu, ops, ctx):
+    """Few sequences with long contexts: one sequence is spread over hundreds of columns of the flat split,
+    so its partial results outnumber the lanes of the combining wave."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    d = W.decode_inputs(ctx, seed=sum(ctx), poison_tail=True)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), f"decode ctx={ctx}")
+
+
 def test_decode_is_bitwise_reproducible(gpu, ops):
     """The same launch repeated gives the same bits: the split of the KV stream over workgroups and the
     order in which partial results are combined do not depend on timing."""
