@@ -139,6 +139,27 @@ int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
                                     void* stream);
 
 /*
+ * The same with the planning step under the caller's control.  The plan (how the KV stream of the batch is
+ * cut over the workgroups) depends only on cache_seqlens, the batch and head counts and the block size, not
+ * on q or on the caches, so the layers of one decode step can share it: call the first layer with
+ * MOPS_HIP_DECODE_PLAN_AND_ATTEND and the others, on the same stream with the same workspace and the same
+ * metadata, with MOPS_HIP_DECODE_REUSE_PLAN.  No counterpart in the reference (its attention call is per layer,
+ * nanovllm/layers/attention.py:40-42).
+ */
+#define MOPS_HIP_DECODE_PLAN_AND_ATTEND 0
+#define MOPS_HIP_DECODE_REUSE_PLAN 1
+int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_stride,
+                                            const void* k_cache, const void* v_cache,
+                                            const int32_t* cache_seqlens,
+                                            const int32_t* block_table, int64_t block_table_row_stride,
+                                            void* out,
+                                            int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                            int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                            float softmax_scale,
+                                            void* workspace, int64_t workspace_bytes,
+                                            int plan_mode, void* stream);
+
+/*
  * Varlen (packed, THD) causal prefill attention with grouped-query heads, with or without a cached prefix.
  * Replaces: flash_attn.flash_attn_varlen_func as reached from mops/torch/ops.py:70-72 and the Triton
  * kernel mops/triton/attention.py:42-146; called at nanovllm/layers/attention.py:34-37 (with the paged

@@ -31,6 +31,10 @@ SIGNATURES = {
                                                 c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                 c_int64, c_int64, c_int64, c_float, c_void_p, c_int64,
                                                 c_void_p]),
+    "mops_hip_attn_paged_decode_planned_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                c_int64, c_int64, c_int64, c_float, c_void_p, c_int64,
+                                                c_int, c_void_p]),
     "mops_hip_attn_varlen_causal_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                                  c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64,
                                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
@@ -44,7 +48,7 @@ SIGNATURES = {
                                             c_int64, c_int64, c_float, c_void_p]),
 }
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib = None
 

@@ -527,19 +527,20 @@ extern "C" int64_t mops_hip_paged_decode_workspace_bytes(int64_t batch, int64_t 
   return workspace_layout(batch, hq, choose_ncols(hkv)).total;
 }
 
-extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
-                                               const void* k_cache, const void* v_cache,
-                                               const int32_t* cache_seqlens,
-                                               const int32_t* block_table, int64_t block_table_row_stride,
-                                               void* out,
-                                               int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
-                                               int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
-                                               float softmax_scale,
-                                               void* workspace, int64_t workspace_bytes,
-                                               void* stream) {
+extern "C" int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_stride,
+                                                       const void* k_cache, const void* v_cache,
+                                                       const int32_t* cache_seqlens,
+                                                       const int32_t* block_table, int64_t block_table_row_stride,
+                                                       void* out,
+                                                       int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                                       int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                                       float softmax_scale,
+                                                       void* workspace, int64_t workspace_bytes,
+                                                       int plan_mode, void* stream) {
   using namespace mops;
   if (batch < 0 || hq <= 0 || hkv <= 0 || block_size <= 0 || num_blocks < 0 || max_blocks_per_seq < 0)
     return MOPS_HIP_EINVAL;
+  if (plan_mode != MOPS_HIP_DECODE_PLAN_AND_ATTEND && plan_mode != MOPS_HIP_DECODE_REUSE_PLAN) return MOPS_HIP_EINVAL;
   if (batch == 0) return MOPS_HIP_OK;
   if (!q || !k_cache || !v_cache || !cache_seqlens || !block_table || !out) return MOPS_HIP_EINVAL;
   if (hq % hkv != 0 || block_table_row_stride < max_blocks_per_seq || num_blocks == 0) return MOPS_HIP_EINVAL;
@@ -588,9 +589,12 @@ extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_st
   p.ws_acc = (float*)(base + w.acc);
   p.ws_ml = (float*)(base + w.ml);
 
-  hipLaunchKernelGGL(paged_decode_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, p);
-  int st = finish_launch();
-  if (st != MOPS_HIP_OK) return st;
+  int st = MOPS_HIP_OK;
+  if (plan_mode != MOPS_HIP_DECODE_REUSE_PLAN) {
+    hipLaunchKernelGGL(paged_decode_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, p);
+    st = finish_launch();
+    if (st != MOPS_HIP_OK) return st;
+  }
 
   const int hpw = choose_hpw(p.hkv);
   const dim3 grid((unsigned)((int64_t)p.ncols * (p.hkv / hpw))), block((unsigned)(kWave * hpw));
@@ -604,4 +608,20 @@ extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_st
   if (st != MOPS_HIP_OK) return st;
   hipLaunchKernelGGL(paged_decode_combine_kernel, dim3((unsigned)(batch * hq)), dim3(kWave), 0, s, p);
   return finish_launch();
+}
+
+extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
+                                               const void* k_cache, const void* v_cache,
+                                               const int32_t* cache_seqlens,
+                                               const int32_t* block_table, int64_t block_table_row_stride,
+                                               void* out,
+                                               int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                               int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                               float softmax_scale,
+                                               void* workspace, int64_t workspace_bytes,
+                                               void* stream) {
+  return mops_hip_attn_paged_decode_planned_bf16(q, q_batch_stride, k_cache, v_cache, cache_seqlens, block_table,
+                                                 block_table_row_stride, out, batch, hq, hkv, head_dim, block_size,
+                                                 num_blocks, max_blocks_per_seq, softmax_scale, workspace, workspace_bytes,
+                                                 MOPS_HIP_DECODE_PLAN_AND_ATTEND, stream);
 }

@@ -83,6 +83,7 @@ class Engine:
         # the fused q_norm + k_norm + rotary + store_kvcache launch, where the backend has it
         self.op_qk_norm_rope_store = mops.get_op("qk_norm_rope_store", backend) if mops.has_op("qk_norm_rope_store", backend) else None
         self.use_fused_qk = True
+        self.share_decode_plan = True   # layers 2..N of a decode step reuse layer 1's split of the KV stream
 
         g = torch.Generator(device=self.dev).manual_seed(seed)
 
@@ -169,8 +170,9 @@ class Engine:
             return self.op_flash_attn_varlen_func(q, k, v, max_seqlen_q=ctx["max_seqlen"], cu_seqlens_q=ctx["cu_seqlens"],
                                                   max_seqlen_k=ctx["max_seqlen"], cu_seqlens_k=ctx["cu_seqlens"],
                                                   softmax_scale=self.scale, causal=True, block_table=None)
+        extra = {"reuse_plan": True} if (self.backend == "hip" and self.share_decode_plan and layer_id > 0) else {}
         return self.op_flash_attn_with_kvcache(q.unsqueeze(1), k_cache, v_cache, cache_seqlens=ctx["context_lens"],
-                                               block_table=ctx["block_tables"], softmax_scale=self.scale, causal=True)
+                                               block_table=ctx["block_tables"], softmax_scale=self.scale, causal=True, **extra)
 
     @torch.inference_mode()
     def forward(self, input_ids, positions, ctx):

@@ -162,8 +162,13 @@ def _decode_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 @register_hip_op
 def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens=None,
-                            block_table=None, softmax_scale=None, causal=True, **kwargs) -> torch.Tensor:
-    """Paged decode attention, q [B, 1, Hq, D] -> [B, 1, Hq, D] (call form: nanovllm/layers/attention.py:40-42)."""
+                            block_table=None, softmax_scale=None, causal=True, reuse_plan: bool = False,
+                            **kwargs) -> torch.Tensor:
+    """Paged decode attention, q [B, 1, Hq, D] -> [B, 1, Hq, D] (call form: nanovllm/layers/attention.py:40-42).
+
+    reuse_plan (extension): skip the planning kernel and use the split the previous call on this stream left
+    in the workspace.  Only valid when that call had the same cache_seqlens, block_table shape and head
+    geometry, i.e. for layers 2..N of one decode step."""
     _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
     _require(cache_seqlens is not None and block_table is not None, "cache_seqlens and block_table are required")
     _require_cuda_bf16("q", q)
@@ -187,12 +192,12 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     lib = _capi.load()
     nbytes = lib.mops_hip_paged_decode_workspace_bytes(batch, hq, hkv, max_blocks, block_size)
     ws = _decode_workspace(q.device, nbytes)
-    st = lib.mops_hip_attn_paged_decode_bf16(q.data_ptr(), q.stride(0) if batch > 1 else hq * d, k_cache.data_ptr(),
-                                             v_cache.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(),
-                                             block_table.stride(0) if batch > 1 else max_blocks, out.data_ptr(),
-                                             batch, hq, hkv, d, block_size, num_blocks, max_blocks, scale,
-                                             ws.data_ptr(), ws.numel(), _stream(q))
-    _capi.check("mops_hip_attn_paged_decode_bf16", st)
+    st = lib.mops_hip_attn_paged_decode_planned_bf16(q.data_ptr(), q.stride(0) if batch > 1 else hq * d, k_cache.data_ptr(),
+                                                     v_cache.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(),
+                                                     block_table.stride(0) if batch > 1 else max_blocks, out.data_ptr(),
+                                                     batch, hq, hkv, d, block_size, num_blocks, max_blocks, scale,
+                                                     ws.data_ptr(), ws.numel(), 1 if reuse_plan else 0, _stream(q))
+    _capi.check("mops_hip_attn_paged_decode_planned_bf16", st)
     return out
 
 

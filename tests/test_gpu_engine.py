@@ -42,8 +42,9 @@ def test_prefill_and_decode_logits_match_oracle_backend(gpu):
 
 
 def test_fused_qk_step_gives_the_same_logits_and_cache_as_the_separate_ops(gpu):
-    """The engine with the fused q_norm/k_norm/rotary/store launch and the same engine with the four separate
-    ops produce bit-identical prefill and decode logits and KV caches."""
+    """The engine with the fused q_norm/k_norm/rotary/store launch and one decode plan per step, and the same
+    engine with the separate ops and a plan per layer, produce bit-identical prefill and decode logits and
+    KV caches."""
     from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
     shape = Qwen3Shape(num_layers=2, vocab=2048)
     g = torch.Generator().manual_seed(5)
@@ -53,6 +54,7 @@ def test_fused_qk_step_gives_the_same_logits_and_cache_as_the_separate_ops(gpu):
         eng = Engine(shape, backend="hip", num_blocks=24, seed=3, device=str(gpu))
         assert eng.op_qk_norm_rope_store is not None
         eng.use_fused_qk = fused
+        eng.share_decode_plan = fused   # and the decode plan shared between the layers, or made per layer
         for p in prompts:
             eng.add_request(p, 4)
         seqs, _ = eng._schedule()

@@ -50,6 +50,20 @@ def test_decode_short_batch_of_long_contexts(gpu, ops, ctx):
     assert_attention_close(_run(hip, d, gpu), _ref(ref, d), f"decode ctx={ctx}")
 
 
+def test_decode_plan_shared_between_calls(gpu, ops):
+    """reuse_plan: a second call with other q and other caches but the same lengths and tables (the next layer
+    of a decode step) skips the planning kernel and gives the bits of a call that plans for itself."""
+    hip, _ = ops("flash_attn_with_kvcache")
+    ctx = W.random_seq_lens(40, 1, 3000, seed=8)
+    d1 = W.to_device(W.decode_inputs(ctx, seed=8), gpu)
+    d2 = W.to_device(W.decode_inputs(ctx, seed=9), gpu)   # same geometry, different data
+    kw = dict(cache_seqlens=d1["cache_seqlens"], block_table=d1["block_table"], softmax_scale=d1["scale"], causal=True)
+    want2 = hip(d2["q"], d2["k_cache"], d2["v_cache"], **kw).clone()
+    hip(d1["q"], d1["k_cache"], d1["v_cache"], **kw)                       # layer 1 plans
+    got2 = hip(d2["q"], d2["k_cache"], d2["v_cache"], reuse_plan=True, **kw)   # layer 2 reuses
+    assert_bit_exact(got2, want2, "decode with a reused plan")
+
+
 def test_decode_is_bitwise_reproducible(gpu, ops):
     """The same launch repeated gives the same bits: the split of the KV stream over workgroups and the
     order in which partial results are combined do not depend on timing."""
