@@ -168,7 +168,7 @@ int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_strid
  *   for sequence s with query tokens [cu_q[s], cu_q[s+1]) and Lk = cu_k[s+1]-cu_k[s] keys (Lk >= Lq):
  *     out[i,h,:] = softmax_{j <= i + (Lk-Lq)}( scale * q[i,h,:] . K_s[j,h/(hq/hkv),:] ) @ V_s[j,h/(hq/hkv),:]
  *
- * q/out: [total_tokens, hq, 128] bf16, token strides in elements, head stride 128.
+ * q/out: [total_tokens, hq, 128] bf16, token strides in elements (multiples of 8), head stride 128.
  * block_table == NULL: k/v are packed [total_k_tokens, hkv, 128] with their own token strides and key j of
  *   sequence s is row cu_k[s] + j; cu_seqlens_k may be NULL (then it equals cu_seqlens_q).
  * block_table != NULL: k/v are the contiguous paged caches [num_blocks, block_size, hkv, 128] and key j of

@@ -92,6 +92,17 @@ __device__ __forceinline__ float half_swap_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// inclusive prefix sum over the 64 lanes of the wave (row shifts, then the two row broadcasts)
+__device__ __forceinline__ int wave_prefix_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // max of three; the compiler fuses the nested form into one v_max3_f32.  It has to stay a compiler-visible
 // operation: the wait states between an MFMA and the first VALU read of its result are inserted by the
 // compiler's hazard recognizer, which does not look inside inline assembly.
@@ -101,6 +112,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPKTile + 2 * kPVTile];  // K[2] then V[2]
+  __shared__ int lds_hist[kPThreads / 64][68];   // per wave: sequences by q tile count (compact launch)
   unsigned char* const lds_k = lds;
   unsigned char* const lds_v = lds + 2 * kPKTile;
 
@@ -143,6 +155,27 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
       const int len = min(qe[j], p.total_tokens) - qs[j];
       cnt[j] = (qs[j] >= 0 && len > 0) ? min((len + kPBM - 1) / kPBM, p.m_tiles) : 0;
     }
+    int r;   // rank of the pair among the sequences that have tile m
+    if (p.m_tiles <= 64) {
+      // Lane l works out how many pairs have a q tile index >= l: a histogram of the sequences by tile
+      // count (this wave's own, in LDS), its prefix sum N(l) = sequences that have tile l, and the prefix
+      // sum of N.  The pair count is non-increasing in l, so one ballot finds the tile index.
+      int* const hist = lds_hist[threadIdx.x >> 6];
+      hist[ln] = 0;
+      if (ln < 4) hist[64 + ln] = 0;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < kPCompactChunks; ++j)
+        if (ln + 64 * j < p.batch) atomicAdd(&hist[cnt[j]], 1);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      const int have = p.batch - wave_prefix_sum(hist[ln]);   // sequences with more than ln tiles
+      const int upto = wave_prefix_sum(have);
+      const int from = __builtin_amdgcn_readlane(upto, 63) - upto + have;   // pairs with q tile index >= ln
+      const unsigned long long reach = __ballot(from > rest);
+      if (reach == 0) return;
+      m = 63 - __builtin_clzll(reach);
+      r = rest - (m < 63 ? __builtin_amdgcn_readlane(from, m + 1) : 0);
+    } else {
     // wave-wide sum of small non-negative integers, one ballot per bit (no trip through LDS)
     const int sum_bits = 32 - __builtin_clz((unsigned)(kPCompactChunks * p.m_tiles));
     auto pairs_from = [&](int mm) {   // pairs whose q tile index is >= mm
@@ -160,7 +193,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
       if (pairs_from(mid) > rest) lo = mid; else hi = mid - 1;
     }
     m = lo;
-    int r = rest - pairs_from(m + 1);   // rank among the sequences that have tile m
+    r = rest - pairs_from(m + 1);
+    }
     b = -1;
     seq_begin = seq_end = kbegin = kend = 0;
 #pragma unroll
@@ -496,10 +530,15 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     }
   }
 
+  // ---- epilogue.  A lane holds 8-byte pieces of its own row, which would make every store instruction
+  //      touch 64 cache lines; the wave's 32 x 128 slab goes through LDS instead and leaves as whole
+  //      256-byte rows, four per store instruction.  The staging area is the K/V buffer pair the last
+  //      tile did not use: no wave reads it any more once all have passed the last tile's barrier.
   l_run = half_swap_sum(l_run);
-  if (my_row < seq_len) {
+  {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    uint16_t* orow = p.out + (int64_t)(seq_begin + my_row) * p.o_ts + (int64_t)h * kPD;
+    constexpr int kOStride = 272;   // bytes between staged rows; 32 rows = half a K buffer
+    unsigned char* const stage = ((wave & 2) ? lds_v + (ntiles & 1) * kPVTile : lds_k + (ntiles & 1) * kPKTile) + (wave & 1) * 32 * kOStride;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -507,8 +546,17 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         u32x2 w;
         w[0] = pack_bf16x2(acc[dt][4 * rq] * inv, acc[dt][4 * rq + 1] * inv);
         w[1] = pack_bf16x2(acc[dt][4 * rq + 2] * inv, acc[dt][4 * rq + 3] * inv);
-        *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * rq + 4 * jj) = w;
+        *reinterpret_cast<u32x2*>(stage + n * kOStride + 64 * dt + 16 * rq + 8 * jj) = w;
       }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes, read back by other lanes
+    const int piece = lane & 15, row4 = lane >> 4;
+    uint16_t* const obase = p.out + (int64_t)(seq_begin + wave_row0) * p.o_ts + (int64_t)h * kPD + 8 * piece;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = row4 + 4 * i;
+      const u32x4 w = *reinterpret_cast<const u32x4*>(stage + row * kOStride + 16 * piece);
+      if (wave_row0 + row < seq_len) *reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts) = w;
+    }
   }
 }
 
@@ -534,7 +582,7 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   if (head_dim != kPD) return MOPS_HIP_EUNSUPPORTED;
   if (q_token_stride < hq * kPD || out_token_stride < hq * kPD) return MOPS_HIP_EINVAL;
   if (total_tokens > 0x3fffffffLL || total_k_tokens > 0x3fffffffLL || batch > (1 << 20) || hq > 4096) return MOPS_HIP_EUNSUPPORTED;
-  if ((q_token_stride & 7) || (out_token_stride & 3)) return MOPS_HIP_EALIGN;
+  if ((q_token_stride & 7) || (out_token_stride & 7)) return MOPS_HIP_EALIGN;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return MOPS_HIP_EALIGN;
   if (block_table) {
     if (!cu_seqlens_k || block_size <= 0 || num_blocks <= 0 || max_blocks_per_seq <= 0 ||
