@@ -37,6 +37,7 @@ def parse_args():
                     choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
+    ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
@@ -53,6 +54,7 @@ def run_e2e(args, torch, dev, mops):
     max_tokens = [random.randint(100, 1024) for _ in range(n)]
     eng = Engine(Qwen3Shape(), backend="hip", num_blocks=max(64, n * 10), seed=args.seed)
     eng.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 8)                 # warm-up, as the reference does
+    eng.pipelined = not args.e2e_stepwise
     if not args.e2e_eager:
         eng.capture_decode_graphs(max_bs=min(512, max(16, (n + 15) // 16 * 16)), max_model_len=4096)
     _, st = eng.generate(prompts, max_tokens, temperature=0.6)
@@ -63,7 +65,8 @@ def run_e2e(args, torch, dev, mops):
         "ms_per_step": round(st["total_s"] * 1e3 / (st["prefill_steps"] + st["decode_steps"]), 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "cfg5 end-to-end generate, random-init Qwen3-0.6B architecture, mops hip backend, decode step "
-                               + ("eager" if args.e2e_eager else "replayed from HIP graphs"),
+                               + ("eager" if args.e2e_eager else "replayed from HIP graphs")
+                               + ("" if args.e2e_eager or args.e2e_stepwise else ", tokens read back once at the end"),
                    "prompts": n, "prompt_len": "uniform[100,1024]", "max_tokens": "uniform[100,1024]", "temperature": 0.6,
                    "output_tokens": total, "prompt_tokens": sum(len(p) for p in prompts)},
         "breakdown": {"seconds": round(st["total_s"], 3), "prefill_steps": st["prefill_steps"], "decode_steps": st["decode_steps"],

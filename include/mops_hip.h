@@ -241,6 +241,38 @@ int mops_hip_qk_norm_rope_store(const void* qkv, int64_t qkv_token_stride, const
                                 void* v_cache, int64_t tokens, int64_t hq, int64_t hkv, int64_t head_dim,
                                 int64_t num_slots, float eps, void* stream);
 
+/*
+ * linear — y = x . W^T (+ bias), bf16 in and out, fp32 accumulation, as a library GEMM (hipBLASLt).
+ * Replaces: mops/torch/ops.py:5-7 (F.linear), called from nanovllm/layers/linear.py:53,75,152 and
+ * nanovllm/layers/embed_head.py:64.
+ * x: [m, k] bf16, w: [n, k] bf16 (nn.Linear layout), y: [m, n] bf16, row strides in elements (% 8 == 0, as
+ * are n and k); bias: [n] bf16 or NULL.  workspace: device scratch for solutions that split k (may be NULL
+ * with workspace_bytes 0; solutions that need more than is given are not chosen).
+ * The solution is the one pinned for (m, n, k) with mops_hip_linear_pin_solution if it supports the
+ * problem, else the first the library's heuristic returns.  Unlike the kernels above this entry point keeps
+ * host-side state (a library handle per device, one descriptor per distinct shape).
+ */
+int mops_hip_linear_bf16(const void* x, int64_t x_row_stride, const void* w, int64_t w_row_stride,
+                         const void* bias, void* y, int64_t y_row_stride,
+                         int64_t m, int64_t n, int64_t k,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Pins the library solution `solution_index` (as returned by mops_hip_linear_tune on the same library
+ * version) for problems with these m, n, k; a negative index removes the pin.  Host-only, no GPU work. */
+int mops_hip_linear_pin_solution(int64_t m, int64_t n, int64_t k, int solution_index);
+
+/*
+ * Times every solution the library offers for (m, n, k) on `distinct_weights` different weight matrices used
+ * in turn (so that none is served from cache, as in a decode step that walks through the layers), `rounds`
+ * passes per measurement, and returns the index of the fastest, its time per GEMM in microseconds, and the
+ * time of the heuristic's choice.  A set-up utility: it allocates and frees its own buffers, creates a
+ * stream and synchronises; not for use on a hot path or under stream capture.  No counterpart in the
+ * reference.
+ */
+int mops_hip_linear_tune(int64_t m, int64_t n, int64_t k, int64_t distinct_weights, int rounds,
+                         void* workspace, int64_t workspace_bytes,
+                         int* best_solution_index, float* best_us, float* heuristic_us);
+
 #ifdef __cplusplus
 }
 #endif

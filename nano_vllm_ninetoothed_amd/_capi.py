@@ -46,9 +46,13 @@ SIGNATURES = {
     "mops_hip_qk_norm_rope_store": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                             c_int64, c_int64, c_float, c_void_p]),
+    "mops_hip_linear_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                     c_int64, c_void_p, c_int64, c_void_p]),
+    "mops_hip_linear_pin_solution": (c_int, [c_int64, c_int64, c_int64, c_int]),
+    "mops_hip_linear_tune": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
 }
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lib = None
 

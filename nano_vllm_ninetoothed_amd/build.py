@@ -73,7 +73,8 @@ def build(force: bool = True, verbose: bool = False) -> Path:
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         objs = list(pool.map(compile_one, srcs))
     tmp = LIB_PATH.with_suffix(".so.tmp")
-    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+    # hipBLASLt is the one library dependency: the `linear` entry point is a library GEMM
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs), "-lhipblaslt"])
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 

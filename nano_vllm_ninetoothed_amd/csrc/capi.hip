@@ -13,7 +13,7 @@ int finish_launch() {
 }
 }  // namespace mops
 
-extern "C" int mops_hip_abi_version(void) { return 6; }
+extern "C" int mops_hip_abi_version(void) { return 7; }
 
 extern "C" int mops_hip_last_hip_error(void) { return mops::g_last_hip_error; }
 

@@ -1,0 +1,261 @@
+// linear: y = x . W^T (+ bias) in bf16 with fp32 accumulation, as a plain library GEMM.
+// Replaces: mops/torch/ops.py:5-7 (F.linear), called from nanovllm/layers/linear.py:53,75,152 and
+// nanovllm/layers/embed_head.py:64.
+//
+// The arithmetic is hipBLASLt's; what this file adds is the choice of the solution.  In a decode step a
+// projection runs on 1..256 rows against weights that no cache holds any more (the 28 layers' weights
+// cycle), and the solution the library's heuristic returns for the shape is not always the one that is
+// fastest there.  A solution can be pinned per (rows, n, k) by its index, and mops_hip_linear_tune finds
+// that index by timing every solution the library offers for the shape on weights that are cold.
+#include "mops_common.h"
+#include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+namespace mops {
+namespace {
+
+struct Problem {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+  bool ready = false;
+};
+
+using Key = std::tuple<int, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int>;   // device, m, n, k, ldx, ldw, ldy, bias
+
+std::mutex g_mu;
+std::map<int, hipblasLtHandle_t> g_handles;                           // per device
+std::map<Key, Problem> g_problems;
+std::map<std::tuple<int64_t, int64_t, int64_t>, int> g_pinned;          // (m, n, k) -> solution index
+
+hipblasLtHandle_t handle_for(int dev) {
+  auto it = g_handles.find(dev);
+  if (it != g_handles.end()) return it->second;
+  hipblasLtHandle_t h = nullptr;
+  if (hipblasLtCreate(&h) != HIPBLAS_STATUS_SUCCESS) return nullptr;
+  g_handles[dev] = h;
+  return h;
+}
+
+// y^T [n x m, column-major] = W [k x n column-major]^T . x^T [k x m column-major]
+bool describe(Problem& p, int64_t m, int64_t n, int64_t k, int64_t ldx, int64_t ldw, int64_t ldy, bool bias) {
+  if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
+  const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+  bool ok = hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)) == HIPBLAS_STATUS_SUCCESS &&
+            hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)) == HIPBLAS_STATUS_SUCCESS;
+  if (ok && bias) {
+    const hipblasLtEpilogue_t ep = HIPBLASLT_EPILOGUE_BIAS;
+    const hipDataType bt = HIP_R_16BF;
+    ok = hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &ep, sizeof(ep)) == HIPBLAS_STATUS_SUCCESS &&
+         hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt)) == HIPBLAS_STATUS_SUCCESS;
+  }
+  ok = ok && hipblasLtMatrixLayoutCreate(&p.la, HIP_R_16BF, k, n, ldw) == HIPBLAS_STATUS_SUCCESS &&
+       hipblasLtMatrixLayoutCreate(&p.lb, HIP_R_16BF, k, m, ldx) == HIPBLAS_STATUS_SUCCESS &&
+       hipblasLtMatrixLayoutCreate(&p.lc, HIP_R_16BF, n, m, ldy) == HIPBLAS_STATUS_SUCCESS;
+  return ok;
+}
+
+void release(Problem& p) {
+  if (p.la) hipblasLtMatrixLayoutDestroy(p.la);
+  if (p.lb) hipblasLtMatrixLayoutDestroy(p.lb);
+  if (p.lc) hipblasLtMatrixLayoutDestroy(p.lc);
+  if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+  p = Problem();
+}
+
+// the pinned solution if there is one and it supports the problem, else the heuristic's first
+bool choose(hipblasLtHandle_t h, Problem& p, int64_t m, int64_t n, int64_t k, size_t workspace_bytes) {
+  const float alpha = 1.f, beta = 0.f;
+  auto pin = g_pinned.find(std::make_tuple(m, n, k));
+  if (pin != g_pinned.end()) {
+    std::vector<int> idx = {pin->second};
+    std::vector<hipblasLtMatmulHeuristicResult_t> found;
+    if (hipblaslt_ext::getAlgosFromIndex(h, idx, found) == HIPBLAS_STATUS_SUCCESS && !found.empty()) {
+      size_t need = 0;
+      if (hipblaslt_ext::matmulIsAlgoSupported(h, p.desc, &alpha, p.la, p.lb, &beta, p.lc, p.lc, found[0].algo, need) == HIPBLAS_STATUS_SUCCESS &&
+          need <= workspace_bytes) {
+        p.algo = found[0].algo;
+        p.workspace = need;
+        return true;
+      }
+    }
+  }
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
+  uint64_t cap = workspace_bytes;
+  hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &cap, sizeof(cap));
+  hipblasLtMatmulHeuristicResult_t res;
+  int got = 0;
+  const auto st = hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, &res, &got);
+  hipblasLtMatmulPreferenceDestroy(pref);
+  if (st != HIPBLAS_STATUS_SUCCESS || got < 1) return false;
+  p.algo = res.algo;
+  p.workspace = res.workspaceSize;
+  return true;
+}
+
+int check_args(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* y, int64_t ldy, int64_t m, int64_t n, int64_t k) {
+  if (m < 0 || n <= 0 || k <= 0) return MOPS_HIP_EINVAL;
+  if (m == 0) return MOPS_HIP_OK;
+  if (!x || !w || !y || ldx < k || ldw < k || ldy < n) return MOPS_HIP_EINVAL;
+  if (m > 0x7fffffffLL || n > 0x7fffffffLL || k > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
+  if (!aligned16(x) || !aligned16(w) || !aligned16(y) || (ldx & 7) || (ldw & 7) || (ldy & 7) || (k & 7) || (n & 7)) return MOPS_HIP_EALIGN;
+  return 1;   // go on
+}
+
+}  // namespace
+}  // namespace mops
+
+extern "C" int mops_hip_linear_bf16(const void* x, int64_t x_row_stride, const void* w, int64_t w_row_stride,
+                                    const void* bias, void* y, int64_t y_row_stride,
+                                    int64_t m, int64_t n, int64_t k,
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
+  using namespace mops;
+  const int pre = check_args(x, x_row_stride, w, w_row_stride, y, y_row_stride, m, n, k);
+  if (pre != 1) return pre;
+  if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return MOPS_HIP_EINVAL;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MOPS_HIP_ELAUNCH;
+  Problem* prob;
+  hipblasLtHandle_t h;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    h = handle_for(dev);
+    if (!h) return MOPS_HIP_ELAUNCH;
+    const Key key{dev, m, n, k, x_row_stride, w_row_stride, y_row_stride, bias ? 1 : 0};
+    prob = &g_problems[key];
+    if (!prob->ready) {
+      if (!describe(*prob, m, n, k, x_row_stride, w_row_stride, y_row_stride, bias != nullptr) ||
+          !choose(h, *prob, m, n, k, (size_t)workspace_bytes)) {
+        release(*prob);
+        g_problems.erase(key);
+        return MOPS_HIP_EUNSUPPORTED;
+      }
+      prob->ready = true;
+    }
+    if (prob->workspace > (size_t)workspace_bytes) return MOPS_HIP_EWORKSPACE;
+    if (bias && hipblasLtMatmulDescSetAttribute(prob->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)) != HIPBLAS_STATUS_SUCCESS)
+      return MOPS_HIP_ELAUNCH;
+    const float alpha = 1.f, beta = 0.f;
+    const auto st = hipblasLtMatmul(h, prob->desc, &alpha, w, prob->la, x, prob->lb, &beta, y, prob->lc, y, prob->lc, &prob->algo,
+                                    workspace, (size_t)workspace_bytes, (hipStream_t)stream);
+    if (st != HIPBLAS_STATUS_SUCCESS) return MOPS_HIP_ELAUNCH;
+  }
+  return finish_launch();
+}
+
+extern "C" int mops_hip_linear_pin_solution(int64_t m, int64_t n, int64_t k, int solution_index) {
+  using namespace mops;
+  if (m <= 0 || n <= 0 || k <= 0) return MOPS_HIP_EINVAL;
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (solution_index < 0) g_pinned.erase(std::make_tuple(m, n, k));
+  else g_pinned[std::make_tuple(m, n, k)] = solution_index;
+  // problems already described for this shape choose again at their next call
+  for (auto it = g_problems.begin(); it != g_problems.end();) {
+    if (std::get<1>(it->first) == m && std::get<2>(it->first) == n && std::get<3>(it->first) == k) {
+      release(it->second);
+      it = g_problems.erase(it);
+    } else {
+      ++it;
+    }
+  }
+  return MOPS_HIP_OK;
+}
+
+extern "C" int mops_hip_linear_tune(int64_t m, int64_t n, int64_t k, int64_t distinct_weights, int rounds,
+                                    void* workspace, int64_t workspace_bytes,
+                                    int* best_solution_index, float* best_us, float* heuristic_us) {
+  using namespace mops;
+  if (m <= 0 || n <= 0 || k <= 0 || distinct_weights <= 0 || rounds <= 0 || !best_solution_index) return MOPS_HIP_EINVAL;
+  if ((k & 7) || (n & 7)) return MOPS_HIP_EALIGN;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MOPS_HIP_ELAUNCH;
+  std::lock_guard<std::mutex> lock(g_mu);
+  hipblasLtHandle_t h = handle_for(dev);
+  if (!h) return MOPS_HIP_ELAUNCH;
+  Problem p;
+  if (!describe(p, m, n, k, k, k, n, false)) { release(p); return MOPS_HIP_EUNSUPPORTED; }
+  void *w = nullptr, *x = nullptr, *y = nullptr;
+  hipStream_t st = nullptr;
+  const size_t w_bytes = (size_t)n * k * 2;
+  int status = MOPS_HIP_OK;
+  if (hipMalloc(&w, w_bytes * distinct_weights) != hipSuccess || hipMalloc(&x, (size_t)m * k * 2) != hipSuccess ||
+      hipMalloc(&y, (size_t)m * n * 2) != hipSuccess || hipStreamCreate(&st) != hipSuccess) {
+    status = MOPS_HIP_ELAUNCH;
+  } else {
+    (void)hipMemsetAsync(w, 0x11, w_bytes * distinct_weights, st);
+    (void)hipMemsetAsync(x, 0x22, (size_t)m * k * 2, st);
+    (void)hipStreamSynchronize(st);
+    const float alpha = 1.f, beta = 0.f;
+    // one pass over all the weights per round, replayed from a graph so that launch cost stays out
+    auto time_algo = [&](hipblasLtMatmulAlgo_t& algo) -> float {
+      hipGraph_t g = nullptr;
+      hipGraphExec_t ge = nullptr;
+      if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess) return -1.f;
+      bool ok = true;
+      for (int r = 0; r < rounds && ok; ++r)
+        for (int64_t l = 0; l < distinct_weights && ok; ++l)
+          ok = hipblasLtMatmul(h, p.desc, &alpha, (const char*)w + l * w_bytes, p.la, x, p.lb, &beta, y, p.lc, y, p.lc, &algo,
+                               workspace, (size_t)workspace_bytes, st) == HIPBLAS_STATUS_SUCCESS;
+      if (hipStreamEndCapture(st, &g) != hipSuccess || !ok || !g) { if (g) (void)hipGraphDestroy(g); return -1.f; }
+      if (hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) != hipSuccess) { (void)hipGraphDestroy(g); return -1.f; }
+      hipEvent_t a, b;
+      (void)hipEventCreate(&a);
+      (void)hipEventCreate(&b);
+      float best = -1.f;
+      if (hipGraphLaunch(ge, st) == hipSuccess && hipStreamSynchronize(st) == hipSuccess) {
+        for (int t = 0; t < 2; ++t) {
+          (void)hipEventRecord(a, st);
+          (void)hipGraphLaunch(ge, st);
+          (void)hipEventRecord(b, st);
+          if (hipStreamSynchronize(st) != hipSuccess) break;
+          float ms = 0.f;
+          (void)hipEventElapsedTime(&ms, a, b);
+          const float us = ms * 1e3f / (float)(rounds * distinct_weights);
+          if (best < 0.f || us < best) best = us;
+        }
+      }
+      (void)hipEventDestroy(a);
+      (void)hipEventDestroy(b);
+      (void)hipGraphExecDestroy(ge);
+      (void)hipGraphDestroy(g);
+      return best;
+    };
+    if (heuristic_us) {
+      *heuristic_us = -1.f;
+      Problem q = p;
+      if (choose(h, q, -1, -1, -1, (size_t)workspace_bytes)) *heuristic_us = time_algo(q.algo);
+    }
+    std::vector<hipblasLtMatmulHeuristicResult_t> all;
+    *best_solution_index = -1;
+    float best = -1.f;
+    if (hipblaslt_ext::getAllAlgos(h, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N, HIP_R_16BF, HIP_R_16BF,
+                                   HIP_R_16BF, HIP_R_16BF, HIPBLAS_COMPUTE_32F, all) == HIPBLAS_STATUS_SUCCESS) {
+      for (auto& cand : all) {
+        size_t need = 0;
+        if (hipblaslt_ext::matmulIsAlgoSupported(h, p.desc, &alpha, p.la, p.lb, &beta, p.lc, p.lc, cand.algo, need) != HIPBLAS_STATUS_SUCCESS ||
+            need > (size_t)workspace_bytes)
+          continue;
+        const float us = time_algo(cand.algo);
+        if (us > 0.f && (best < 0.f || us < best)) {
+          best = us;
+          *best_solution_index = hipblaslt_ext::getIndexFromAlgo(cand.algo);
+        }
+      }
+    }
+    if (best_us) *best_us = best;
+    if (*best_solution_index < 0) status = MOPS_HIP_EUNSUPPORTED;
+  }
+  if (st) (void)hipStreamDestroy(st);
+  if (w) (void)hipFree(w);
+  if (x) (void)hipFree(x);
+  if (y) (void)hipFree(y);
+  release(p);
+  return status;
+}

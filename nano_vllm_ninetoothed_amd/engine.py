@@ -14,6 +14,11 @@ What it mirrors (and nothing more):
     max_num_batched_tokens / max_num_seqs, otherwise one decode step for every running sequence.
   * optional HIP-graph replay of the decode forward for bucketed batch sizes with static input buffers,
     slot_mapping padded with -1 and context_lens with 0 (model_runner.py:189-206, 216-251).
+Beyond the reference: with graphs captured, generate() does not wait for a step's tokens before it issues
+the next step.  Which sequences run, their lengths, slots and block tables depend only on token counts, so
+the host prepares step t+1 while the GPU works on step t; the sampled tokens stay on the device (one row
+per sequence, gathered as the next step's input ids) and are read back once at the end.  The reference
+reads them back every step (model_runner.py:212), which leaves the GPU idle while the host schedules.
 Not mirrored: prefix caching, preemption (the cache is sized so it never triggers), tensor parallelism,
 the tokenizer, weight loading.
 
@@ -55,6 +60,8 @@ class Sequence:
     temperature: float
     num_prompt_tokens: int = 0
     block_table: list = field(default_factory=list)
+    row: int = -1      # pipelined generation: this sequence's row in the device-side last-token table
+    filled: int = 0    # pipelined generation: completion tokens whose values have been read back
 
     def __post_init__(self):
         self.num_prompt_tokens = len(self.token_ids)
@@ -117,6 +124,12 @@ class Engine:
         self.scale = s.head_dim ** -0.5
         self.graphs = {}
         self.graph_bs = []
+        # pipelined generation (see the module docstring): last sampled token per sequence row; row 0
+        # takes the writes of padding rows
+        self.pipelined = True
+        self.last_tok = torch.zeros(max_num_seqs + 1, dtype=torch.int64, device=self.dev)
+        self.free_rows = deque(range(1, max_num_seqs + 1))
+        self.unit_temps = torch.ones(max_num_seqs, dtype=torch.float32, device=self.dev)
 
     # ------------------------------------------------------------------ HIP graphs for decode
     @torch.inference_mode()
@@ -127,10 +140,19 @@ class Engine:
         max_blocks = (max_model_len + BLOCK_SIZE - 1) // BLOCK_SIZE
         dev = self.dev
         self.g_ids = torch.zeros(max_bs, dtype=torch.int64, device=dev)
-        self.g_pos = torch.zeros(max_bs, dtype=torch.int64, device=dev)
-        self.g_slots = torch.full((max_bs,), -1, dtype=torch.int32, device=dev)
-        self.g_lens = torch.zeros(max_bs, dtype=torch.int32, device=dev)
-        self.g_tables = torch.full((max_bs, max_blocks), -1, dtype=torch.int32, device=dev)
+        self.g_i64 = torch.zeros((2, max_bs), dtype=torch.int64, device=dev)    # int64 copies of rows and positions
+        self.g_rows64, self.g_pos = self.g_i64[0], self.g_i64[1]
+        # the int32 inputs are views of one buffer, so that one host-to-device copy can fill them all:
+        # [sequence rows | positions | slots | lengths | block tables]
+        self.g_meta = torch.empty(max_bs * (4 + max_blocks), dtype=torch.int32, device=dev)
+        self.g_rows, self.g_pos32 = self.g_meta[:max_bs], self.g_meta[max_bs:2 * max_bs]
+        self.g_slots, self.g_lens = self.g_meta[2 * max_bs:3 * max_bs], self.g_meta[3 * max_bs:4 * max_bs]
+        self.g_tables = self.g_meta[4 * max_bs:].view(max_bs, max_blocks)
+        self.g_rows.zero_()
+        self.g_pos32.zero_()
+        self.g_slots.fill_(-1)
+        self.g_lens.zero_()
+        self.g_tables.fill_(-1)
         self.g_out = torch.zeros((max_bs, self.shape.hidden), dtype=torch.bfloat16, device=dev)
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
         pool = None
@@ -159,7 +181,8 @@ class Engine:
         self.g_lens[:bs] = ctx["context_lens"]
         self.g_tables[:bs, : ctx["block_tables"].size(1)] = ctx["block_tables"]
         self.graphs[bucket].replay()
-        return self.op_linear(self.g_out[:bs], self.embed)
+        # the lm head runs on the bucket's row count, like the captured layers: GEMM solutions are chosen per shape
+        return self.op_linear(self.g_out[:bucket], self.embed)[:bs]
 
     # ------------------------------------------------------------------ model
     def _attention(self, layer_id, q, k, v, ctx, stored=False):
@@ -291,6 +314,109 @@ class Engine:
             q.block_table = []
         return seqs, is_prefill, finished
 
+    @torch.inference_mode()
+    def _generate_pipelined(self, stats):
+        """Runs until no sequence is waiting or running without reading a token back in between."""
+        import numpy as np
+        dev = self.dev
+        n, max_blocks = self.g_ids.numel(), self.g_tables.size(1)
+        depth = 8                                  # steps the host may be ahead of the GPU
+        staging = [torch.empty(self.g_meta.numel(), dtype=torch.int32, pin_memory=True) for _ in range(depth)]
+        staged = [None] * depth                    # event: the copy out of that staging buffer has run
+        hist_rows = 2048
+        hist = torch.empty((hist_rows, self.max_num_seqs), dtype=torch.int64, device=dev)
+        steps = []                                 # (history row, sequences, is_prefill, end-of-step event)
+        mark = torch.cuda.Event(enable_timing=True)
+        mark.record()
+
+        def drain():
+            nonlocal mark
+            if not steps:
+                return
+            torch.cuda.synchronize(dev)
+            host = hist[:len(steps)].cpu()
+            prev = mark
+            for h, seqs, is_prefill, ev in steps:
+                row = host[h].tolist()
+                for j, q in enumerate(seqs):
+                    q.token_ids[q.num_prompt_tokens + q.filled] = row[j]
+                    q.filled += 1
+                stats["prefill_s" if is_prefill else "decode_s"] += prev.elapsed_time(ev) * 1e-3
+                prev = ev
+            mark = prev
+            steps.clear()
+
+        it = 0
+        while self.waiting or self.running:
+            if len(steps) == hist_rows:
+                drain()
+            seqs, is_prefill = self._schedule()
+            bs = len(seqs)
+            graphable = (not is_prefill and bs <= self.graph_bs[-1]
+                         and max(len(q.block_table) for q in seqs) <= max_blocks)
+            if is_prefill:
+                if len(self.free_rows) < bs:     # more sequences in flight than rows so far: grow the table
+                    old = self.last_tok.numel()
+                    self.last_tok = torch.cat((self.last_tok, torch.zeros(max(bs, old), dtype=torch.int64, device=dev)))
+                    self.free_rows.extend(range(old, self.last_tok.numel()))
+                for q in seqs:
+                    q.row = self.free_rows.popleft()
+                ids, pos, ctx = self._prepare_prefill(seqs)
+                logits = self.forward(ids, pos, ctx)
+                rows = self._to_dev([q.row for q in seqs], torch.int64)
+            elif graphable:
+                slot = it % depth
+                it += 1
+                if staged[slot] is not None:
+                    staged[slot].synchronize()
+                a = staging[slot].numpy()
+                a[:2 * n] = 0
+                a[2 * n:3 * n] = -1
+                a[3 * n:4 * n] = 0
+                a[4 * n:] = -1
+                a[:bs] = [q.row for q in seqs]
+                a[n:n + bs] = [len(q) - 1 for q in seqs]
+                a[2 * n:2 * n + bs] = [q.block_table[-1] * BLOCK_SIZE + (len(q) - 1) % BLOCK_SIZE for q in seqs]
+                a[3 * n:3 * n + bs] = [len(q) for q in seqs]
+                tab = a[4 * n:].reshape(n, max_blocks)
+                for j, q in enumerate(seqs):
+                    tab[j, :len(q.block_table)] = q.block_table
+                self.g_meta.copy_(staging[slot], non_blocking=True)
+                staged[slot] = torch.cuda.Event()
+                staged[slot].record()
+                bucket = next(b for b in self.graph_bs if b >= bs)
+                self.g_i64.copy_(self.g_meta[:2 * n].view(2, n))
+                torch.index_select(self.last_tok, 0, self.g_rows64[:bucket], out=self.g_ids[:bucket])
+                self.graphs[bucket].replay()
+                logits = self.op_linear(self.g_out[:bucket], self.embed)[:bs]
+                rows = self.g_rows64[:bs]
+            else:                                   # a batch no graph covers: this step runs the stepwise way
+                drain()
+                ids, pos, ctx = self._prepare_decode(seqs)
+                logits = self.forward(ids, pos, ctx)
+                rows = self._to_dev([q.row for q in seqs], torch.int64)
+            tok = self.op_sampler_forward(logits, self.unit_temps[:bs])   # greedy: the temperature does not move the argmax
+            self.last_tok.index_copy_(0, rows, tok)
+            hist[len(steps), :bs] = tok
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            steps.append((len(steps), list(seqs), is_prefill, ev))
+            for q in seqs:
+                q.token_ids.append(-1)              # value pending; only the count matters to the scheduler
+                if q.num_completion_tokens >= q.max_tokens:
+                    self.running.remove(q)
+                    self.free_blocks.extend(q.block_table)
+                    q.block_table = []
+                    self.free_rows.append(q.row)
+                    q.row = -1
+            if is_prefill:
+                stats["prefill_steps"] += 1
+                stats["prefill_tokens"] += sum(len(q) - 1 for q in seqs)
+            else:
+                stats["decode_steps"] += 1
+                stats["decode_tokens"] += bs
+        drain()
+
     def generate(self, prompts, max_tokens, temperature=0.6):
         """prompts: list of token-id lists; max_tokens: int or list.  Returns (completions, stats)."""
         if isinstance(max_tokens, int):
@@ -302,7 +428,9 @@ class Engine:
         stats = dict(prefill_steps=0, decode_steps=0, prefill_tokens=0, decode_tokens=0, prefill_s=0.0, decode_s=0.0)
         torch.cuda.synchronize(self.dev)
         t_all = time.perf_counter()
-        while self.waiting or self.running:
+        if self.graphs and self.pipelined:
+            self._generate_pipelined(stats)
+        while self.waiting or self.running:     # stepwise: every step's tokens are read back before the next
             t0 = time.perf_counter()
             seqs, is_prefill, _ = self.step()
             dt = time.perf_counter() - t0

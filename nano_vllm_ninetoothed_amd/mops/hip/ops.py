@@ -1,6 +1,6 @@
 """The `hip` backend: the six hot operators, plus siluAndMul, apply_rotary_emb and sampler_forward, run
-hand-written gfx950 kernels through the C ABI of libmops_hip.so; linear and softmax are library-torch
-delegates so that the engine's layers resolve.
+hand-written gfx950 kernels through the C ABI of libmops_hip.so; linear is a library GEMM (hipBLASLt through
+the same C ABI for the decode-sized problems, torch otherwise) and softmax a library-torch delegate.
 
 Every function keeps the name and call form the reference's layers use (nanovllm/layers/attention.py:29-42,
 layernorm.py:21,29, embed_head.py:41).  Wrappers validate layouts with exceptions before launching
@@ -261,8 +261,67 @@ def flash_attn_varlen_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ma
 # and softmax are library torch on the GPU, as in mops/torch/ops.py:5-7,37-43
 # ----------------------------------------------------------------------------------------------------
 
+_LINEAR_MAX_ROWS = 1024          # above this the GEMM is compute-bound and goes to the library through torch
+_LINEAR_WORKSPACE_BYTES = 32 << 20
+_linear_workspaces: dict = {}
+_linear_pins_loaded = False
+
+
+def _linear_workspace(device: torch.device) -> torch.Tensor:
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _linear_workspaces.get(key)
+    if ws is None:
+        ws = torch.empty(_LINEAR_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _linear_workspaces[key] = ws
+    return ws
+
+
+def load_linear_solutions(path=None) -> int:
+    """Pins the hipBLASLt solutions listed in a file written by `python -m nano_vllm_ninetoothed_amd.tune_linear`
+    (default: the table shipped in the package, measured on MI355X).  A table made with another library
+    version is ignored: solution indices do not carry over.  Returns the number of shapes pinned."""
+    import json
+    from pathlib import Path
+    path = Path(path) if path is not None else Path(__file__).resolve().parents[2] / "data" / "linear_solutions_gfx950.json"
+    if not path.exists():
+        return 0
+    table = json.loads(path.read_text())
+    if table.get("hip_version") != torch.version.hip:
+        return 0
+    lib = _capi.load()
+    for m, n, k, index in table["solutions"]:
+        _capi.check("mops_hip_linear_pin_solution", lib.mops_hip_linear_pin_solution(m, n, k, index))
+    return len(table["solutions"])
+
+
 @register_hip_op
 def linear(x, weight, bias=None):
+    """x @ weight.T (+ bias) (mops/torch/ops.py:5-7).  A library GEMM either way: bf16 problems with up to
+    1024 rows (the decode step's projections, the lm head) call hipBLASLt through the C ABI, which lets a
+    solution measured on cold weights be pinned per shape; everything else goes through torch."""
+    global _linear_pins_loaded
+    if (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.dim() == 2
+            and weight.stride(1) == 1 and x.dim() >= 1 and x.shape[-1] == weight.shape[1]
+            and (bias is None or (bias.dtype == torch.bfloat16 and bias.is_contiguous() and bias.numel() == weight.shape[0]))):
+        n, k = weight.shape
+        x2 = x.reshape(-1, k)
+        if x2.stride(1) != 1:
+            x2 = x2.contiguous()
+        m = x2.shape[0]
+        ldx = x2.stride(0) if m > 1 else k
+        ldw = weight.stride(0) if n > 1 else k
+        if (0 < m <= _LINEAR_MAX_ROWS and k % 8 == 0 and n % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0
+                and x2.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and (bias is None or bias.data_ptr() % 16 == 0)):
+            if not _linear_pins_loaded:
+                _linear_pins_loaded = True
+                load_linear_solutions()
+            y = torch.empty((m, n), dtype=x.dtype, device=x.device)
+            ws = _linear_workspace(x.device)
+            st = _capi.load().mops_hip_linear_bf16(x2.data_ptr(), ldx, weight.data_ptr(), ldw,
+                                                   bias.data_ptr() if bias is not None else None, y.data_ptr(), n, m, n, k,
+                                                   ws.data_ptr(), ws.numel(), _stream(x))
+            _capi.check("mops_hip_linear_bf16", st)
+            return y.view(*x.shape[:-1], n)
     return torch.nn.functional.linear(x, weight, bias)
 
 

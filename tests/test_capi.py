@@ -105,3 +105,17 @@ def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
     monkeypatch.setattr(_capi, "LIB_PATH", tmp_path / "libmops_hip.so")
     with pytest.raises(ImportError):
         _capi.load()
+
+
+def test_linear_argument_validation(lib):
+    """linear: validation happens on the host before the GEMM library is touched."""
+    A = 0x1000
+    assert lib.mops_hip_linear_bf16(A, 1024, A, 1024, None, A, 4096, 0, 4096, 1024, None, 0, None) == 0       # no rows
+    assert lib.mops_hip_linear_bf16(None, 1024, A, 1024, None, A, 4096, 4, 4096, 1024, None, 0, None) == -1
+    assert lib.mops_hip_linear_bf16(A, 512, A, 1024, None, A, 4096, 4, 4096, 1024, None, 0, None) == -1    # x stride < k
+    assert lib.mops_hip_linear_bf16(A, 1024, A, 1024, None, A, 4096, 4, 4096, 1020, None, 0, None) == -3   # k % 8
+    assert lib.mops_hip_linear_bf16(A, 1024, A, 1024, None, A + 2, 4096, 4, 4096, 1024, None, 0, None) == -3
+    assert lib.mops_hip_linear_bf16(A, 1024, A, 1024, None, A, 4096, 4, 4096, 1024, None, 64, None) == -1     # bytes without a pointer
+    assert lib.mops_hip_linear_pin_solution(0, 4096, 1024, 5) == -1
+    assert lib.mops_hip_linear_pin_solution(4, 4096, 1024, 5) == 0 and lib.mops_hip_linear_pin_solution(4, 4096, 1024, -1) == 0
+    assert lib.mops_hip_linear_tune(0, 4096, 1024, 28, 1, None, 0, None, None, None) == -1

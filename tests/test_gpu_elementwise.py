@@ -118,3 +118,54 @@ def test_fused_qk_norm_rope_store_equals_the_separate_ops(gpu, tokens, hq, hkv, 
     assert (q_f.float().cpu() - q_o.float()).abs().max() <= 0.0625
     assert_bit_exact(vc_f, vc_o, "v cache vs oracle")
     assert ((kc_f.float().cpu() - kc_o.float()).abs() <= 0.0625).all()
+
+
+@pytest.mark.parametrize("m,n,k,bias", [(256, 4096, 1024, False), (1, 1024, 2048, False), (37, 6144, 1024, True),
+                                        (512, 1024, 3072, False), (16, 2048, 1024, True)])
+def test_linear_matches_fp32_reference(gpu, m, n, k, bias):
+    """linear through the C ABI (a library GEMM with fp32 accumulation) against x.float() @ w.float().T in
+    fp32: the only error allowed is the bf16 rounding of the result and the order of the fp32 sums."""
+    from nano_vllm_ninetoothed_amd import mops
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(gpu)
+    w = (torch.randn(n, k, generator=g) * k ** -0.5).to(torch.bfloat16).to(gpu)
+    b = torch.randn(n, generator=g).to(torch.bfloat16).to(gpu) if bias else None
+    y = mops.linear(x, w, b)
+    assert y.shape == (m, n) and y.dtype == torch.bfloat16
+    ref = x.float() @ w.float().t()
+    if bias:
+        ref = ref + b.float()
+    err = (y.float() - ref).abs()
+    assert err.max().item() <= 2 ** -7 * ref.abs().max().item() + 1e-3
+    # a strided input (a column slice of a wider buffer) and leading dimensions
+    wide = torch.randn(2, max(m // 2, 1), k + 64, generator=g).to(torch.bfloat16).to(gpu)
+    xs = wide[..., 32:32 + k]
+    ys = mops.linear(xs, w, b)
+    refs = xs.float() @ w.float().t() + (b.float() if bias else 0)
+    assert ys.shape == (2, max(m // 2, 1), n)
+    assert (ys.float() - refs).abs().max().item() <= 2 ** -7 * refs.abs().max().item() + 1e-3
+
+
+def test_linear_with_a_pinned_solution_and_tuning(gpu):
+    """mops_hip_linear_tune returns a solution index for a small shape; pinning it keeps the result within
+    the same bound, and removing the pin goes back to the heuristic's choice."""
+    import ctypes
+    from nano_vllm_ninetoothed_amd import _capi, mops
+    lib = _capi.load()
+    m, n, k = 16, 256, 512
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(gpu)
+    w = (torch.randn(n, k, generator=g) * k ** -0.5).to(torch.bfloat16).to(gpu)
+    ref = x.float() @ w.float().t()
+    y0 = mops.linear(x, w)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=gpu)
+    best, best_us, heur_us = ctypes.c_int(-1), ctypes.c_float(-1), ctypes.c_float(-1)
+    st = lib.mops_hip_linear_tune(m, n, k, 2, 1, ws.data_ptr(), ws.numel(), ctypes.byref(best), ctypes.byref(best_us), ctypes.byref(heur_us))
+    assert st == 0 and best.value >= 0 and best_us.value > 0 and heur_us.value > 0
+    assert lib.mops_hip_linear_pin_solution(m, n, k, best.value) == 0
+    y1 = mops.linear(x, w)
+    assert lib.mops_hip_linear_pin_solution(m, n, k, -1) == 0
+    y2 = mops.linear(x, w)
+    for y in (y0, y1, y2):
+        assert (y.float() - ref).abs().max().item() <= 2 ** -7 * ref.abs().max().item() + 1e-3
+    assert torch.equal(y0, y2)

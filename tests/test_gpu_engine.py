@@ -98,10 +98,46 @@ def test_graph_replay_matches_eager_decode(gpu):
         seqs, is_prefill = eng._schedule()
         assert not is_prefill
         ids, pos, ctx = eng._prepare_decode(seqs)
-        eager = eng.forward(ids, pos, ctx)
+        # eager run on the same padded batch the graph sees (the GEMM library picks its kernels by row count)
+        bs, bucket = len(seqs), 8
+        pad = bucket - bs
+        ids_p = torch.cat((ids, ids.new_zeros(pad)))
+        pos_p = torch.cat((pos, pos.new_zeros(pad)))
+        ctx_p = dict(is_prefill=False, slot_mapping=torch.cat((ctx["slot_mapping"], ctx["slot_mapping"].new_full((pad,), -1))),
+                     context_lens=torch.cat((ctx["context_lens"], ctx["context_lens"].new_zeros(pad))),
+                     block_tables=torch.cat((ctx["block_tables"], ctx["block_tables"].new_full((pad, ctx["block_tables"].size(1)), -1))))
+        eager = eng.forward(ids_p, pos_p, ctx_p)[:bs]
         torch.cuda.synchronize()
         replay = eng._decode_replay(ids, pos, ctx)
         torch.cuda.synchronize()
         assert torch.equal(eager, replay), f"replay {it} differs from eager"
         for q in seqs:
             q.token_ids.append(int(eager[0].argmax()) % 2048)
+
+
+def test_pipelined_generate_gives_the_tokens_of_stepwise_generate(gpu):
+    """generate() with graphs captured keeps the sampled tokens on the device and reads them back at the
+    end; the tokens, the step counts and the freed state must equal those of the stepwise loop, which reads
+    every step's tokens back before it schedules the next.  Run twice on the same engine: the second call
+    starts from the rows and blocks the first one freed."""
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    shape = Qwen3Shape(num_layers=2, vocab=2048)
+    g = torch.Generator().manual_seed(9)
+    res = []
+    for pipelined in (True, False):
+        eng = Engine(shape, backend="hip", num_blocks=64, seed=4, device=str(gpu), max_num_seqs=8, max_num_batched_tokens=1024)
+        eng.capture_decode_graphs(max_bs=16, max_model_len=1024)
+        eng.pipelined = pipelined
+        runs = []
+        for rnd in range(2):
+            gg = torch.Generator().manual_seed(20 + rnd)
+            lens = (40, 300, 255, 256, 7, 130, 1, 90, 64, 200, 33)          # more prompts than max_num_seqs
+            prompts = [torch.randint(0, 2048, (n,), generator=gg).tolist() for n in lens]
+            max_tokens = [5, 12, 1, 7, 30, 2, 9, 16, 3, 21, 8]
+            outs, stats = eng.generate(prompts, max_tokens)
+            assert [len(o) for o in outs] == max_tokens
+            assert all(0 <= t < 2048 for o in outs for t in o)
+            assert len(eng.free_blocks) == 64 and not eng.running and not eng.waiting
+            runs.append((outs, stats["prefill_steps"], stats["decode_steps"], stats["decode_tokens"]))
+        res.append(runs)
+    assert res[0] == res[1]
