@@ -76,6 +76,13 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: the hip backend has no fallback. Build it with "
             "`python -m nano_vllm_ninetoothed_amd.build` (needs hipcc, no GPU required)."
         )
+    try:
+        # torch wheels carry their own HIP runtime and hipBLASLt under the sonames this library links
+        # against; importing torch first keeps one copy of each in the process, whichever order the caller
+        # imports things in (and the GEMM solution table was measured against that copy)
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(str(LIB_PATH))
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError here means header and library disagree

@@ -279,14 +279,15 @@ def _linear_workspace(device: torch.device) -> torch.Tensor:
 def load_linear_solutions(path=None) -> int:
     """Pins the hipBLASLt solutions listed in a file written by `python -m nano_vllm_ninetoothed_amd.tune_linear`
     (default: the table shipped in the package, measured on MI355X).  A table made with another library
-    version is ignored: solution indices do not carry over.  Returns the number of shapes pinned."""
+    version or for another GPU architecture is ignored: solution indices do not carry over.  Returns the number of shapes pinned."""
     import json
     from pathlib import Path
     path = Path(path) if path is not None else Path(__file__).resolve().parents[2] / "data" / "linear_solutions_gfx950.json"
     if not path.exists():
         return 0
     table = json.loads(path.read_text())
-    if table.get("hip_version") != torch.version.hip:
+    arch = torch.cuda.get_device_properties(torch.cuda.current_device()).gcnArchName.split(":")[0]
+    if table.get("hip_version") != torch.version.hip or table.get("arch") != arch:
         return 0
     lib = _capi.load()
     for m, n, k, index in table["solutions"]:

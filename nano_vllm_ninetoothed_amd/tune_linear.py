@@ -17,6 +17,18 @@ import sys
 import time
 
 
+def _dump(table: dict) -> str:
+    """JSON with one table entry per line."""
+    head = {k: v for k, v in table.items() if k not in ("solutions", "timings_us")}
+    lines = ["{"] + [f'"{k}": {json.dumps(v)},' for k, v in head.items()]
+    for key in ("solutions", "timings_us"):
+        lines.append(f'"{key}": [')
+        lines += [json.dumps(e) + ("," if i + 1 < len(table[key]) else "") for i, e in enumerate(table[key])]
+        lines.append("]," if key == "solutions" else "]")
+    lines.append("}")
+    return "\n".join(lines) + "\n"
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", required=True)
@@ -34,11 +46,13 @@ def main() -> int:
     ws = torch.empty(32 << 20, dtype=torch.uint8, device=dev)
     shapes = [tuple(int(v) for v in s.split(":")) for s in args.shapes.split(",")]
     rows = [int(r) for r in args.rows.split(",")]
-    out = {"hip_version": torch.version.hip, "device": torch.cuda.get_device_name(0), "solutions": [], "timings_us": []}
+    out = {"hip_version": torch.version.hip, "arch": torch.cuda.get_device_properties(dev).gcnArchName.split(":")[0],
+           "note": "hipBLASLt solution index per [rows, n, k], fastest on cold weights; timings_us rows are [rows, n, k, best, heuristic's choice]",
+           "solutions": [], "timings_us": []}
     if args.merge and os.path.exists(args.out):
         with open(args.out) as f:
             old = json.load(f)
-        if old.get("hip_version") == out["hip_version"]:
+        if old.get("hip_version") == out["hip_version"] and old.get("arch") == out["arch"]:
             todo = {(m, n, k) for m in rows for n, k in shapes}
             out["solutions"] = [e for e in old["solutions"] if tuple(e[:3]) not in todo]
             out["timings_us"] = [e for e in old["timings_us"] if tuple(e[:3]) not in todo]
@@ -54,7 +68,7 @@ def main() -> int:
             print(f"m={m} n={n} k={k}: solution {best.value} {best_us.value:.2f} us (heuristic's choice {heur_us.value:.2f} us), "
                   f"searched in {time.time() - t0:.1f} s", flush=True)
             with open(args.out, "w") as f:      # rewritten after every shape so that a cut-off run still leaves a table
-                json.dump(out, f, indent=0)
+                f.write(_dump(out))
     return 0
 
 
