@@ -49,6 +49,18 @@ def test_prefill_many_ragged_sequences(gpu, ops, nseq):
     assert_attention_close(_run(hip, d, gpu), _ref(ref, d), f"prefill {nseq} ragged sequences")
 
 
+def test_prefill_ragged_batch_with_a_very_long_sequence(gpu, ops):
+    """More than 64 q tiles in the longest sequence: the rank -> (tile, sequence) mapping of the compact
+    launch takes its search form instead of the one-ballot form.  Two query heads keep the oracle quick."""
+    hip, ref = ops("flash_attn_varlen_func")
+    lens = [150, 8400, 0, 64, 129, 1]
+    d = W.prefill_inputs(lens, hq=2, hkv=1, seed=84)
+    want = _ref(ref, d)
+    assert_attention_close(_run(hip, d, gpu), want, "ragged batch with an 8400-token sequence")
+    # and the same lengths when max_seqlen_q is a loose bound (more tile indices than any sequence has)
+    assert_attention_close(_run(hip, d, gpu, max_seqlen_q=16384), want, "same, max_seqlen_q = 16384")
+
+
 def test_prefill_v_is_strided_view_and_max_seqlen_is_only_a_bound(gpu, ops):
     """q, k, v as nanovllm hands them: slices of one [T, 4096] qkv buffer (row stride 4096)."""
     hip, ref = ops("flash_attn_varlen_func")
