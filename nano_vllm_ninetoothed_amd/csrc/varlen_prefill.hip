@@ -6,7 +6,8 @@
 //   rows 32w..32w+31; two workgroups per CU.  Tiles with the longest causal prefix are dispatched first,
 //   and with 8 kv heads the workgroup id is decoded so that id % 8 — the XCD a workgroup lands on — is
 //   the kv head: each XCD's L2 then only ever holds one kv head's K/V.  Ragged batches launch workgroups
-//   for existing q tiles only (the kernel maps the workgroup's rank to its tile and sequence).
+//   for existing q tiles only (the kernel maps the workgroup's rank to its tile and sequence).  The output
+//   slab of a wave leaves through LDS as whole 256-byte rows.
 //
 // Per 64-token K/V tile (double-buffered in LDS, one workgroup barrier per tile), hand scheduled: every
 // MFMA opens a slot, and what the wave issues while that MFMA runs is fixed by scheduling fences
@@ -43,6 +44,10 @@
 //     8192-token sequences, -10 % on 128..2048-token ones), one wave per SIMD owning two 32-row slabs
 //     (512 registers; the compiler shuttles values between the two register files), software-pipelining
 //     the two products across half tiles inside a wave (register pressure, two barriers per tile).
+//   * Per workgroup there is a fixed cost of ~7 us next to ~2 us per tile: rank -> tile mapping, Q and
+//     first-tile loads, the epilogue, and the gap until the dispatcher starts the successor.  A persistent
+//     launch (resident workgroups drawing items by ticket) did not shrink it (it is dependent latency, not
+//     dispatch time) and lengthened the tail; it was 6 % slower on 128..2048-token sequences.
 //   * The transposing read ds_read_b64_tr_b16 delivers ~65 B/clk per CU against ~210 B/clk for
 //     ds_read_b128, but replacing it by plain reads of a pre-transposed tile changed the run time by
 //     2 %: the LDS pipe is not what bounds this shape.
