@@ -175,6 +175,48 @@ def test_decode_full_size_properties(gpu, ops, hq, hkv, lo, hi, bsz):
     assert_attention_close(got[pick], _ref(ref, sub), "sampled sequences of the full-size batch")
 
 
+def test_decode_8b_shape_full_size_properties(gpu, ops):
+    """The 8B-shaped benchmark configuration at full size (512 sequences, 32 query / 8 kv heads, contexts
+    1024..8192, ~9.7 GB of cache) with the cache filled on the device: finiteness, the convex-hull bound
+    |o| <= max|v|, and a sample of sequences checked against the oracle on a cache cut down to their blocks."""
+    hip, ref = ops("flash_attn_with_kvcache")
+    bsz, hq, hkv, bs = 512, 32, 8, 256
+    ctx = torch.tensor(W.random_seq_lens(bsz, 1024, 8192, seed=0), dtype=torch.int64)
+    nblocks = (ctx + bs - 1) // bs
+    total = int(nblocks.sum())
+    g = torch.Generator().manual_seed(4)
+    perm = torch.randperm(total, generator=g).to(torch.int32)
+    table = torch.full((bsz, int(nblocks.max())), -1, dtype=torch.int32)
+    pos = 0
+    for b in range(bsz):
+        table[b, :int(nblocks[b])] = perm[pos:pos + int(nblocks[b])]
+        pos += int(nblocks[b])
+    gd = torch.Generator(device=gpu).manual_seed(4)
+    k_cache = torch.empty((total, bs, hkv, 128), dtype=torch.bfloat16, device=gpu)
+    v_cache = torch.empty_like(k_cache)
+    for r in range(0, total, 512):      # filled in slabs: the fp32 draw of the whole cache would not fit beside it
+        n = min(512, total - r)
+        k_cache[r:r + n] = torch.randn((n, bs, hkv, 128), generator=gd, device=gpu, dtype=torch.float32).to(torch.bfloat16)
+        v_cache[r:r + n] = torch.randn((n, bs, hkv, 128), generator=gd, device=gpu, dtype=torch.float32).to(torch.bfloat16)
+    q = torch.randn((bsz, 1, hq, 128), generator=g).to(torch.bfloat16)
+    scale = 128 ** -0.5
+    got = hip(q.to(gpu), k_cache, v_cache, cache_seqlens=ctx.to(torch.int32).to(gpu), block_table=table.to(gpu),
+              softmax_scale=scale, causal=True)
+    assert got.shape == (bsz, 1, hq, 128)
+    assert torch.isfinite(got.float()).all()
+    assert got.float().abs().max() <= v_cache.float().abs().max()
+    pick = [0, 7, 255, 511, int(ctx.argmax()), int(ctx.argmin())]
+    blocks = torch.cat([table[b, :int(nblocks[b])] for b in pick]).long()
+    sub_table = torch.full((len(pick), table.shape[1]), -1, dtype=torch.int32)
+    pos = 0
+    for i, b in enumerate(pick):
+        sub_table[i, :int(nblocks[b])] = torch.arange(pos, pos + int(nblocks[b]), dtype=torch.int32)
+        pos += int(nblocks[b])
+    want = ref(q[pick], k_cache[blocks.to(gpu)].cpu(), v_cache[blocks.to(gpu)].cpu(), cache_seqlens=ctx[pick].to(torch.int32),
+               block_table=sub_table, softmax_scale=scale, causal=True)
+    assert_attention_close(got[pick].cpu(), want, "sampled sequences of the 8B-shaped full-size batch")
+
+
 @pytest.mark.parametrize("ctx,hq,hkv", [([300, 900, 31], 8, 4), ([700, 5], 4, 2), ([513, 1025], 16, 1), ([2000], 12, 6)])
 def test_decode_other_head_counts(gpu, ops, ctx, hq, hkv):
     hip, ref = ops("flash_attn_with_kvcache")
