@@ -34,7 +34,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
+                    choices=["decode", "decode8b", "prefill", "prefill_long", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
@@ -195,8 +195,10 @@ def main():
             return (sorted(ts)[len(ts) // 2], f"first {n} of {bsz} sequences, median of {len(ts)} passes (~12 s of CPU work)",
                     W.decode_bytes(ctx[:n], hq, hkv, max_blocks))
 
-    elif args.op == "prefill":
-        lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
+    elif args.op in ("prefill", "prefill_long"):
+        # prefill_long: four 8192-token sequences, where the fixed cost per 128-row item no longer shows
+        long_case = args.op == "prefill_long"
+        lens = [8192] * 4 if long_case else W.random_seq_lens(16, 128, 2048, seed=args.seed)
         d = W.to_device(W.prefill_inputs(lens, seed=args.seed), dev)
         op = mops.flash_attn_varlen_func
 
@@ -207,8 +209,10 @@ def main():
         work = W.prefill_flops(lens, 16)
         bound = "mfma"
         metric, unit = "varlen_prefill_attn_TFLOPs", "TFLOP/s"
-        config = {"workload": "cfg2 varlen causal prefill, Qwen3-0.6B shape", "batch": 16, "q_heads": 16, "kv_heads": 8,
-                  "head_dim": 128, "seq_lens": f"uniform[128,2048] seed {args.seed}", "total_tokens": sum(lens)}
+        config = {"workload": ("varlen causal prefill, four 8192-token sequences, Qwen3-0.6B shape" if long_case
+                               else "cfg2 varlen causal prefill, Qwen3-0.6B shape"), "batch": len(lens), "q_heads": 16, "kv_heads": 8,
+                  "head_dim": 128, "seq_lens": "4 x 8192" if long_case else f"uniform[128,2048] seed {args.seed}",
+                  "total_tokens": sum(lens)}
         kernel_name = "varlen_prefill_kernel"
 
         def cpu_fn():
@@ -216,6 +220,11 @@ def main():
             ref = mops.get_op("flash_attn_varlen_func", "torch")
             c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
             ts = []
+            if long_case:   # one 8192-token sequence is ~10 s of CPU work; the batch is four of them
+                one = {"q": c["q"][:8192], "k": c["k"][:8192], "v": c["v"][:8192], "cu": c["cu_seqlens"][:2]}
+                t0 = time.perf_counter()
+                ref(one["q"], one["k"], one["v"], max_seqlen_q=8192, cu_seqlens_q=one["cu"], softmax_scale=c["scale"])
+                return time.perf_counter() - t0, "first of the four sequences, one run", work / 4
             for _ in range(3):
                 t0 = time.perf_counter()
                 ref(c["q"], c["k"], c["v"], max_seqlen_q=c["max_seqlen"], cu_seqlens_q=c["cu_seqlens"], softmax_scale=c["scale"])
