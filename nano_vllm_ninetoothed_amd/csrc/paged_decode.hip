@@ -41,7 +41,13 @@ constexpr int kRowBytes = kHeadDim * 2;                  // one token, one kv he
 constexpr int kTileBytes = kStageTokens * kRowBytes;     // 8 KiB
 constexpr int kPlanThreads = 256;
 constexpr int kPlanLdsSeqs = 4096;                       // prefix array kept in LDS up to this batch
-constexpr int kHdrInts = 64;                             // workspace header: [0] total stages, [1] stages per column
+constexpr int kHdrInts = 64;                             // workspace header, see PlanHeader
+// Header words.  [2..8] are the signature of the launch the plan was made for: a kernel that is handed
+// a workspace whose plan does not fit its own parameters (never planned, or planned for another batch or
+// head geometry) must not follow it, because the sequence indices in it would be out of range.
+enum PlanHeader { kHdrTotal = 0, kHdrPerCol = 1, kHdrMagic = 2, kHdrBatch = 3, kHdrCols = 4, kHdrHq = 5, kHdrHkv = 6,
+                  kHdrBlockSize = 7, kHdrMaxBlocks = 8 };
+constexpr int kPlanMagic = 0x6d6f7073;
 
 // Byte offset of 16-byte piece `slice` of token row `t` inside a swizzled LDS tile.
 __device__ __forceinline__ int tile_offset(int t, int slice) {
@@ -74,6 +80,14 @@ __device__ __forceinline__ int clamp_seqlen(int s, const DecodeParams& p) {
   return s < 0 ? 0 : (s > cap ? cap : s);
 }
 __device__ __forceinline__ int stages_of(int seqlen) { return (seqlen + kStageTokens - 1) / kStageTokens; }
+
+// True when the plan in the workspace was made for a launch with these parameters.
+__device__ __forceinline__ bool plan_fits(const DecodeParams& p) {
+  const int32_t* h = p.hdr;
+  return h[kHdrMagic] == kPlanMagic && h[kHdrBatch] == p.batch && h[kHdrCols] == p.ncols && h[kHdrHq] == p.hq &&
+         h[kHdrHkv] == p.hkv && h[kHdrBlockSize] == p.block_size && h[kHdrMaxBlocks] == p.max_blocks_per_seq &&
+         h[kHdrPerCol] > 0 && h[kHdrTotal] >= 0;
+}
 
 // Scalar (constant-cache) load of a wave-uniform int that no kernel in flight writes.  Used inside
 // the main loop, where a vector load would have to wait behind the whole queue of KV loads.
@@ -120,8 +134,15 @@ __global__ __launch_bounds__(kPlanThreads) void paged_decode_plan_kernel(const D
   }
   const int per_col = max(p.min_per_col, (total + p.ncols - 1) / p.ncols);
   if (tid == 0) {
-    p.hdr[0] = total;
-    p.hdr[1] = per_col;
+    p.hdr[kHdrTotal] = total;
+    p.hdr[kHdrPerCol] = per_col;
+    p.hdr[kHdrMagic] = kPlanMagic;
+    p.hdr[kHdrBatch] = p.batch;
+    p.hdr[kHdrCols] = p.ncols;
+    p.hdr[kHdrHq] = p.hq;
+    p.hdr[kHdrHkv] = p.hkv;
+    p.hdr[kHdrBlockSize] = p.block_size;
+    p.hdr[kHdrMaxBlocks] = p.max_blocks_per_seq;
   }
   __syncthreads();
   const int* pre = use_lds ? prefix_lds : p.prefix;
@@ -168,8 +189,9 @@ __global__ __launch_bounds__(kWave * HPW, 2) void paged_decode_kernel(const Deco
   const int n_hg = p.hkv / HPW;                      // head groups (workgroups) per column
   const int col = blockIdx.x / n_hg;
   const int g = (blockIdx.x % n_hg) * HPW + wave;    // this wave's kv head
-  const int total = p.hdr[0];
-  const int per_col = p.hdr[1];
+  if (!plan_fits(p)) return;   // the combine kernel writes zero rows in that case
+  const int total = p.hdr[kHdrTotal];
+  const int per_col = p.hdr[kHdrPerCol];
   const int64_t flat0 = (int64_t)col * per_col;
   if (flat0 >= total) return;
   int remaining = min(per_col, total - (int)flat0);  // stages left in this column's run
@@ -244,8 +266,10 @@ __global__ __launch_bounds__(kWave * HPW, 2) void paged_decode_kernel(const Deco
     }
   };
 
-  Piece cur = make_piece(p.col_start[2 * col], p.col_start[2 * col + 1], remaining);
-  if (!cur.valid) return;  // cannot happen for a planned run
+  const int b_first = p.col_start[2 * col], s_first = p.col_start[2 * col + 1];
+  if (b_first < 0 || b_first >= p.batch || s_first < 0) return;   // cannot happen for a planned run
+  Piece cur = make_piece(b_first, s_first, remaining);
+  if (!cur.valid) return;  // a plan made for other lengths: nothing of this sequence lies in the run
 
   bf16x8 qb[4];
   f32x4 acc[8];
@@ -423,12 +447,16 @@ __global__ __launch_bounds__(kWave) void paged_decode_combine_kernel(const Decod
   const int b = bh / p.hq;
   const int h = bh % p.hq;
   const int lane = threadIdx.x;
-  const int f0 = p.prefix[b], f1 = p.prefix[b + 1];
-  if (f1 == f0) {  // an empty context attends to nothing: zeros
+  if (!plan_fits(p)) {  // no usable plan: the main kernel did nothing; leave a defined (zero) row
     reinterpret_cast<uint32_t*>(p.out + (int64_t)bh * kHeadDim)[lane] = 0u;
     return;
   }
-  const int per_col = p.hdr[1];
+  const int f0 = p.prefix[b], f1 = p.prefix[b + 1];
+  if (f1 <= f0) {  // an empty context attends to nothing: zeros
+    reinterpret_cast<uint32_t*>(p.out + (int64_t)bh * kHeadDim)[lane] = 0u;
+    return;
+  }
+  const int per_col = p.hdr[kHdrPerCol];
   const int j0 = f0 / per_col, j1 = (f1 - 1) / per_col;
   if (j0 == j1) return;  // one piece: written directly by the main kernel
   // partial of column j: slot 1 in the column where the sequence begins, slot 0 in the following ones
@@ -527,17 +555,19 @@ extern "C" int64_t mops_hip_paged_decode_workspace_bytes(int64_t batch, int64_t 
   return workspace_layout(batch, hq, choose_ncols(hkv)).total;
 }
 
-extern "C" int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_stride,
-                                                       const void* k_cache, const void* v_cache,
-                                                       const int32_t* cache_seqlens,
-                                                       const int32_t* block_table, int64_t block_table_row_stride,
-                                                       void* out,
-                                                       int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
-                                                       int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
-                                                       float softmax_scale,
-                                                       void* workspace, int64_t workspace_bytes,
-                                                       int plan_mode, void* stream) {
-  using namespace mops;
+namespace mops {
+
+// Validates the arguments and launches plan (unless reused), main and combine kernels with `workspace` as scratch.
+static int launch_paged_decode(const void* q, int64_t q_batch_stride,
+                               const void* k_cache, const void* v_cache,
+                               const int32_t* cache_seqlens,
+                               const int32_t* block_table, int64_t block_table_row_stride,
+                               void* out,
+                               int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                               int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                               float softmax_scale,
+                               void* workspace, int64_t workspace_bytes,
+                               int plan_mode, void* stream) {
   if (batch < 0 || hq <= 0 || hkv <= 0 || block_size <= 0 || num_blocks < 0 || max_blocks_per_seq < 0)
     return MOPS_HIP_EINVAL;
   if (plan_mode != MOPS_HIP_DECODE_PLAN_AND_ATTEND && plan_mode != MOPS_HIP_DECODE_REUSE_PLAN) return MOPS_HIP_EINVAL;
@@ -608,6 +638,23 @@ extern "C" int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_
   if (st != MOPS_HIP_OK) return st;
   hipLaunchKernelGGL(paged_decode_combine_kernel, dim3((unsigned)(batch * hq)), dim3(kWave), 0, s, p);
   return finish_launch();
+}
+
+}  // namespace mops
+
+extern "C" int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_stride,
+                                                       const void* k_cache, const void* v_cache,
+                                                       const int32_t* cache_seqlens,
+                                                       const int32_t* block_table, int64_t block_table_row_stride,
+                                                       void* out,
+                                                       int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                                       int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                                       float softmax_scale,
+                                                       void* workspace, int64_t workspace_bytes,
+                                                       int plan_mode, void* stream) {
+  return mops::launch_paged_decode(q, q_batch_stride, k_cache, v_cache, cache_seqlens, block_table, block_table_row_stride,
+                                   out, batch, hq, hkv, head_dim, block_size, num_blocks, max_blocks_per_seq, softmax_scale,
+                                   workspace, workspace_bytes, plan_mode, stream);
 }
 
 extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,

@@ -133,10 +133,11 @@ class Engine:
 
     # ------------------------------------------------------------------ HIP graphs for decode
     @torch.inference_mode()
-    def capture_decode_graphs(self, max_bs: int = 256, max_model_len: int = 4096):
+    def capture_decode_graphs(self, max_bs: int = 256, max_model_len: int = 4096, smallest_first: bool = False):
         """Captures the decode forward (embedding .. final norm) once per batch-size bucket.  Replays
         read their inputs from static buffers; rows beyond the live batch carry slot -1 / length 0,
-        which store_kvcache skips and paged decode answers with zeros."""
+        which store_kvcache skips and paged decode answers with zeros.  The order of the captures does not matter
+        (smallest_first exists for the test of that)."""
         max_blocks = (max_model_len + BLOCK_SIZE - 1) // BLOCK_SIZE
         dev = self.dev
         self.g_ids = torch.zeros(max_bs, dtype=torch.int64, device=dev)
@@ -155,14 +156,22 @@ class Engine:
         self.g_tables.fill_(-1)
         self.g_out = torch.zeros((max_bs, self.shape.hidden), dtype=torch.bfloat16, device=dev)
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
+        # Every bucket is captured on one stream of our own.  The ops keep their scratch buffers per stream, and
+        # the graphs hold those addresses: sizing the scratch for the largest bucket on that stream before the
+        # first capture means no capture, in whatever order, allocates or moves it.
+        capture_stream = torch.cuda.Stream(dev)
+        if self.backend == "hip":
+            from .mops.hip.ops import reserve_decode_workspace
+            with torch.cuda.stream(capture_stream):
+                reserve_decode_workspace(max_bs, self.shape.num_heads, self.shape.num_kv_heads, max_blocks, BLOCK_SIZE, dev)
         pool = None
-        for bs in reversed(self.graph_bs):
+        for bs in (self.graph_bs if smallest_first else reversed(self.graph_bs)):
             ctx = dict(is_prefill=False, slot_mapping=self.g_slots[:bs], context_lens=self.g_lens[:bs],
                        block_tables=self.g_tables[:bs], hidden_only=True)
             graph = torch.cuda.CUDAGraph()
             self.g_out[:bs] = self.forward(self.g_ids[:bs], self.g_pos[:bs], ctx)      # warm-up outside capture
             torch.cuda.synchronize(dev)
-            with torch.cuda.graph(graph, pool):
+            with torch.cuda.graph(graph, pool, stream=capture_stream):
                 self.g_out[:bs] = self.forward(self.g_ids[:bs], self.g_pos[:bs], ctx)
             if pool is None:
                 pool = graph.pool()

@@ -146,18 +146,44 @@ def add_rms_forward(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tenso
     return y, r_out
 
 
-_workspaces: dict = {}
+_workspaces: dict = {}          # (device index, stream handle) -> current scratch tensor
+_retired_workspaces: list = []  # superseded scratch tensors: captured graphs may still hold their addresses
+_last_plan: dict = {}           # (device index, stream handle) -> description of the plan the scratch holds
+
+
+def _workspace_key(device: torch.device):
+    return (device.index if device.index is not None else torch.cuda.current_device(),
+            torch.cuda.current_stream(device).cuda_stream)
 
 
 def _decode_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Per-(device, stream) scratch for split-context partials; grown on demand, reused across calls
-    on the same stream (kernels on one stream run in order, so reuse cannot race)."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    """Per-(device, stream) scratch for split-context partials, reused across calls on the same stream
+    (kernels on one stream run in order, so reuse cannot race).  It grows on demand; a buffer that has been
+    handed out is never freed, because a captured HIP graph replays with the address it was captured with.
+    Callers that capture graphs size it once with reserve_decode_workspace() before the first capture."""
+    key = _workspace_key(device)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            _retired_workspaces.append(ws)
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
+        _last_plan.pop(key, None)
     return ws
+
+
+def reserve_decode_workspace(max_batch: int, hq: int, hkv: int, max_blocks: int, block_size: int = 256,
+                             device=None) -> int:
+    """Sizes the current stream's paged-decode scratch (scratch is kept per stream: make the stream that will
+    capture current first) for problems of up to max_batch sequences, so that no later
+    flash_attn_with_kvcache call on this stream with at most that many sequences allocates (the scratch size grows
+    with the batch only).  Call it before capturing HIP graphs: captures of any batch size, in any order, then
+    share one buffer that stays where it is.  Returns the size in bytes."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    nbytes = _capi.load().mops_hip_paged_decode_workspace_bytes(max_batch, hq, hkv, max_blocks, block_size)
+    _require(nbytes > 0, "reserve_decode_workspace: sizes must be positive")
+    _linear_workspace(device)   # the GEMM scratch of this stream has a fixed size; make it exist as well
+    return _decode_workspace(device, nbytes).numel()
 
 
 @register_hip_op
@@ -166,9 +192,10 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             **kwargs) -> torch.Tensor:
     """Paged decode attention, q [B, 1, Hq, D] -> [B, 1, Hq, D] (call form: nanovllm/layers/attention.py:40-42).
 
-    reuse_plan (extension): skip the planning kernel and use the split the previous call on this stream left
-    in the workspace.  Only valid when that call had the same cache_seqlens, block_table shape and head
-    geometry, i.e. for layers 2..N of one decode step."""
+    reuse_plan (extension): skip the planning kernel and use the split the last planning call on this stream left
+    in the scratch.  Only valid when that call had the same cache_seqlens and block_table tensors and the same
+    head geometry, i.e. for layers 2..N of one decode step; anything else raises ValueError.  (The kernels
+    themselves refuse a plan whose recorded batch or head geometry differs from their launch and write zeros.)"""
     _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
     _require(cache_seqlens is not None and block_table is not None, "cache_seqlens and block_table are required")
     _require_cuda_bf16("q", q)
@@ -192,6 +219,15 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     lib = _capi.load()
     nbytes = lib.mops_hip_paged_decode_workspace_bytes(batch, hq, hkv, max_blocks, block_size)
     ws = _decode_workspace(q.device, nbytes)
+    # what the plan in the scratch depends on; a reused plan must have been made for exactly this
+    plan = (ws.data_ptr(), batch, hq, hkv, block_size, cache_seqlens.data_ptr(), block_table.data_ptr(), tuple(block_table.shape))
+    key = _workspace_key(q.device)
+    if reuse_plan:
+        _require(_last_plan.get(key) == plan,
+                 "reuse_plan=True, but the last planning call on this stream was made for another batch, head geometry, "
+                 "cache_seqlens or block_table (or there was none)")
+    else:
+        _last_plan[key] = plan
     st = lib.mops_hip_attn_paged_decode_planned_bf16(q.data_ptr(), q.stride(0) if batch > 1 else hq * d, k_cache.data_ptr(),
                                                      v_cache.data_ptr(), cache_seqlens.data_ptr(), block_table.data_ptr(),
                                                      block_table.stride(0) if batch > 1 else max_blocks, out.data_ptr(),

@@ -82,9 +82,12 @@ def test_generate_respects_max_tokens_and_frees_blocks(gpu):
     assert stats["prefill_steps"] == 1 and stats["decode_steps"] == 9
 
 
-def test_graph_replay_matches_eager_decode(gpu):
+@pytest.mark.parametrize("smallest_first", [False, True])
+def test_graph_replay_matches_eager_decode(gpu, smallest_first):
     """The captured decode forward is replayed several times with eager work and synchronisation in
-    between; every replay must reproduce the eager logits bit for bit, including with padded rows."""
+    between; every replay must reproduce the eager logits bit for bit, including with padded rows.  With
+    smallest_first the small buckets are captured before the large ones: the attention scratch the graphs point
+    at is sized before the first capture, so a later, larger capture must not move it."""
     from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
     shape = Qwen3Shape(num_layers=2, vocab=2048)
     eng = Engine(shape, backend="hip", num_blocks=40, seed=5, device=str(gpu))
@@ -93,7 +96,7 @@ def test_graph_replay_matches_eager_decode(gpu):
     for p in prompts:
         eng.add_request(p, 64)
     eng.step()                                    # prefill
-    eng.capture_decode_graphs(max_bs=16, max_model_len=1024)
+    eng.capture_decode_graphs(max_bs=16, max_model_len=1024, smallest_first=smallest_first)
     for it in range(4):
         seqs, is_prefill = eng._schedule()
         assert not is_prefill
@@ -141,3 +144,10 @@ def test_pipelined_generate_gives_the_tokens_of_stepwise_generate(gpu):
             runs.append((outs, stats["prefill_steps"], stats["decode_steps"], stats["decode_tokens"]))
         res.append(runs)
     assert res[0] == res[1]
+
+
+def test_shipped_gemm_solution_table_is_applied(gpu):
+    """The table of hipBLASLt solutions shipped in the package was measured for this GPU and this library
+    version; if either differs the loader pins nothing and the engine silently runs on the heuristic's picks."""
+    from nano_vllm_ninetoothed_amd.mops.hip.ops import load_linear_solutions
+    assert load_linear_solutions() > 0

@@ -277,3 +277,49 @@ def test_decode_other_block_sizes(gpu, ops, block_size):
         got = hip(d2["q"].to(gpu), kc.to(gpu), vc.to(gpu), cache_seqlens=d2["cache_seqlens"].to(gpu), block_table=tbl.to(gpu),
                   softmax_scale=d2["scale"], causal=True)
         assert_attention_close(got, want, "block size 512")
+
+
+def test_reuse_plan_without_a_matching_plan_is_refused(gpu, ops):
+    """reuse_plan=True is only legal right after a planning call with the same metadata tensors and head
+    geometry on the same stream; the wrapper raises instead of launching on a plan made for something else."""
+    hip, _ = ops("flash_attn_with_kvcache")
+    d1 = W.to_device(W.decode_inputs([700, 300, 64], seed=31), gpu)
+    d2 = W.to_device(W.decode_inputs([700, 300, 64, 90], seed=32), gpu)
+    kw1 = dict(cache_seqlens=d1["cache_seqlens"], block_table=d1["block_table"], softmax_scale=d1["scale"], causal=True)
+    kw2 = dict(cache_seqlens=d2["cache_seqlens"], block_table=d2["block_table"], softmax_scale=d2["scale"], causal=True)
+    hip(d1["q"], d1["k_cache"], d1["v_cache"], **kw1)
+    with pytest.raises(ValueError, match="reuse_plan"):
+        hip(d2["q"], d2["k_cache"], d2["v_cache"], reuse_plan=True, **kw2)        # other batch, other tensors
+    with pytest.raises(ValueError, match="reuse_plan"):
+        hip(d1["q"], d1["k_cache"], d1["v_cache"], reuse_plan=True, **dict(kw1, cache_seqlens=d1["cache_seqlens"].clone()))
+    hip(d1["q"], d1["k_cache"], d1["v_cache"], reuse_plan=True, **kw1)            # the matching one is accepted
+
+
+def test_kernels_refuse_a_plan_made_for_another_launch(gpu):
+    """Through the C ABI, where nothing tracks the plan: MOPS_HIP_DECODE_REUSE_PLAN on a workspace that was never
+    planned, or was planned for a larger batch, must not follow the stale sequence indices.  The kernels compare the
+    plan's recorded batch and head geometry with their own launch and write zero rows instead."""
+    from nano_vllm_ninetoothed_amd import _capi
+    lib = _capi.load()
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+    big = W.to_device(W.decode_inputs(W.random_seq_lens(64, 1, 2000, seed=33), seed=33), gpu)
+    small = W.to_device(W.decode_inputs([500, 900, 40], seed=34), gpu)
+
+    def call(g, ws, mode):
+        q, kc, bt = g["q"], g["k_cache"], g["block_table"]
+        out = torch.full_like(q, float("nan"))
+        st = lib.mops_hip_attn_paged_decode_planned_bf16(
+            q.data_ptr(), q.stride(0), kc.data_ptr(), g["v_cache"].data_ptr(), g["cache_seqlens"].data_ptr(), bt.data_ptr(),
+            bt.stride(0), out.data_ptr(), q.shape[0], q.shape[2], kc.shape[2], 128, kc.shape[1], kc.shape[0], bt.shape[1],
+            g["scale"], ws.data_ptr(), ws.numel(), mode, stream)
+        _capi.check("mops_hip_attn_paged_decode_planned_bf16", st)
+        torch.cuda.synchronize()
+        return out
+
+    nbytes = lib.mops_hip_paged_decode_workspace_bytes(64, 16, 8, 16, 256)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=gpu)
+    assert (call(small, ws, 1).float() == 0).all(), "never planned"
+    want_small = call(small, ws.clone(), 0)
+    call(big, ws, 0)                                                   # plan for 64 sequences
+    assert (call(small, ws, 1).float() == 0).all(), "planned for a larger batch"
+    assert_bit_exact(call(small, ws, 0), want_small, "planning afresh on the used workspace")
