@@ -20,6 +20,12 @@ What pins each function (all in tests/test_oracle.py, none of it a retyped copy 
   flash_attn_with_kvcache        fp64 brute force; equals the last row of causal prefill over the same
                                  K/V; invariant under a joint permutation of cache blocks and block_table;
                                  NaN sentinels beyond cache_seqlens do not reach the output.
+  apply_rotary_emb               complex multiplication in fp64; identity at angle 0 and the quarter turn
+                                 (x1, x2) -> (-x2, x1), both bit for bit; pair-norm preservation; R(t)R(-t) = I.
+  siluAndMul                     fp64 x / (1 + e^-x) with the two bf16 roundings; the single-rounding variant differs.
+  sampler_forward                brute-force first-maximum loop, with ties, the last column and an all-equal row.
+  qk_norm_rope_store             fp64 loops on a tiny input with norm weights that vary along the head, so that
+                                 rotary-before-norm fails; raw v and rotated k in their slots; slot -1 skipped.
 The rounding internal to flash-attn itself (P cast to bf16 before PV, exp2 softmax) is pinned by no file
 available here: attention parity is therefore stated with the tolerance max-abs 2e-2 / mean-abs 2e-3.
 """

@@ -216,3 +216,134 @@ def test_prefix_prefill_against_fp64_brute_force_and_packed_form(O):
     plain = O.flash_attn_varlen_func(d["q"][lo:hi], d["k_all"][klo:klo + 3], d["v_all"][klo:klo + 3], max_seqlen_q=3,
                                      cu_seqlens_q=torch.tensor([0, 3], dtype=torch.int32), softmax_scale=d["scale"], causal=True)
     assert_bit_exact(paged[lo:hi], plain, "empty prefix")
+
+
+# ------------------------------------------------------------------------------------------ ops beside the six
+# (apply_rotary_emb, siluAndMul, sampler_forward and the fused q/k front end: the GPU tests of those kernels
+# compare against these oracle functions, so they are pinned here by what the mathematics fixes)
+
+def _rotary_case(tokens=5, heads=3, d=16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((tokens, heads, d), generator=g).to(torch.bfloat16)
+    theta = torch.rand((tokens, 1, d // 2), generator=g, dtype=torch.float64) * 6.0 - 3.0
+    return x, theta
+
+
+def test_rotary_is_complex_multiplication(O):
+    """mops/torch/ops.py:45-54: with z = x1 + i*x2 (first and second half of the head), y = z * e^{i*theta}."""
+    x, theta = _rotary_case(seed=1)
+    got = O.apply_rotary_emb(x, theta.cos().float(), theta.sin().float())
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    half = x.shape[-1] // 2
+    z = torch.complex(x[..., :half].double(), x[..., half:].double()) * torch.polar(torch.ones_like(theta), theta)
+    want = torch.cat((z.real, z.imag), dim=-1)
+    d = ulp_distance_bf16(got, want.float().to(torch.bfloat16))
+    assert int(d.max()) <= 1 and (d == 0).float().mean() > 0.98   # fp32 cos/sin and products against fp64
+
+
+def test_rotary_special_angles_and_inverse(O):
+    x, theta = _rotary_case(tokens=4, heads=2, d=32, seed=2)
+    half = x.shape[-1] // 2
+    one, zero = torch.ones_like(theta).float(), torch.zeros_like(theta).float()
+    # position 0: cos 1, sin 0 -> identity, bit for bit
+    assert_bit_exact(O.apply_rotary_emb(x, one, zero), x, "rotation by 0")
+    # quarter turn: (x1, x2) -> (-x2, x1) exactly; a swapped sign or swapped halves fails here
+    q = O.apply_rotary_emb(x, zero, one)
+    assert_bit_exact(q[..., :half], -x[..., half:], "quarter turn, first half")
+    assert_bit_exact(q[..., half:], x[..., :half], "quarter turn, second half")
+    # a rotation preserves the length of every (x1[i], x2[i]) pair, and rotating back undoes it (bf16 roundings apart)
+    c, s = theta.cos().float(), theta.sin().float()
+    y = O.apply_rotary_emb(x, c, s)
+    n_x = x[..., :half].double() ** 2 + x[..., half:].double() ** 2
+    n_y = y[..., :half].double() ** 2 + y[..., half:].double() ** 2
+    assert torch.allclose(n_x, n_y, rtol=2 ** -6, atol=1e-6)
+    back = O.apply_rotary_emb(y, c, -s)
+    assert (back.double() - x.double()).abs().max() <= 2 ** -6 * x.double().abs().max()
+
+
+def test_silu_and_mul_against_fp64(O):
+    """mops/torch/ops.py:32-34: F.silu(x) * y on bf16 tensors = bf16(bf16(x / (1 + e^-x)) * y)."""
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn((64, 96), generator=g) * 3).to(torch.bfloat16)
+    y = torch.randn((64, 96), generator=g).to(torch.bfloat16)
+    x[0, :4] = torch.tensor([0.0, -0.0, 30.0, -30.0], dtype=torch.bfloat16)
+    got = O.siluAndMul(x, y)
+    silu = np.array([[v / (1.0 + math.exp(-v)) for v in row] for row in x.double().tolist()])
+    first = to_bf16_from_f64(silu)                                     # first rounding
+    want = to_bf16_from_f64(first.double().numpy() * y.double().numpy())  # second rounding
+    d = ulp_distance_bf16(got, want)
+    assert int(d.max()) <= 1 and (d == 0).float().mean() > 0.995
+    assert got[0, 0] == 0 and got[0, 1] == 0                           # silu(0) = 0
+    assert got[0, 2] == (torch.tensor(30.0, dtype=torch.bfloat16) * y[0, 2])  # silu(30) = 30 to bf16 precision
+    # the first rounding is really there: silu(x) * y from an unrounded silu differs somewhere
+    single = to_bf16_from_f64(silu * y.double().numpy())
+    assert not torch.equal(single, want)
+
+
+def test_sampler_is_first_index_of_the_largest_logit(O):
+    """mops/torch/ops.py:37-43 with the Gumbel line commented out: argmax(softmax(logits / T)); for T > 0 that is
+    the index of the largest logit, the first one on exact ties."""
+    g = torch.Generator().manual_seed(4)
+    logits = (torch.randn((12, 257), generator=g) * 4).to(torch.bfloat16)
+    logits[1, 200] = logits[1, 17] = logits[1].max() + 1           # a tie: the first index wins
+    logits[2, 256] = 50.0                                          # the last column
+    logits[3, :] = -3.0                                            # all equal: index 0
+    temps = torch.rand(12, generator=g) * 2 + 0.05
+    got = O.sampler_forward(logits, temps)
+    assert got.dtype == torch.int64 and got.shape == (12,)
+    want = []
+    for row in logits.double().tolist():
+        best, arg = -math.inf, -1
+        for i, v in enumerate(row):
+            if v > best:
+                best, arg = v, i
+        want.append(arg)
+    assert got.tolist() == want
+    assert got[1] == 17 and got[2] == 256 and got[3] == 0
+
+
+def test_fused_qk_front_end_is_norm_then_rotary_then_store(O):
+    """nanovllm/models/qwen3.py:74-80 + nanovllm/layers/attention.py:29-31 in fp64 loops on a tiny input: per-head
+    RMSNorm of q and k (weight applied after the first rounding), THEN the rotation, the rotated k and the raw v
+    written to the slot.  The norm weights vary strongly along the head, so the other order fails."""
+    g = torch.Generator().manual_seed(5)
+    T, hq, hkv, d, eps = 3, 2, 1, 8, 1e-6
+    half = d // 2
+    qkv = torch.randn((T, (hq + 2 * hkv) * d), generator=g).to(torch.bfloat16)
+    qw = torch.linspace(0.25, 4.0, d).to(torch.bfloat16)
+    kw = torch.linspace(3.0, 0.5, d).to(torch.bfloat16)
+    theta = torch.rand((T, 1, half), generator=g, dtype=torch.float64) * 3
+    cos, sin = theta.cos().float(), theta.sin().float()
+    k_cache = torch.full((2, 4, hkv, d), 7.0, dtype=torch.bfloat16)
+    v_cache = torch.full((2, 4, hkv, d), 7.0, dtype=torch.bfloat16)
+    slots = torch.tensor([5, -1, 2], dtype=torch.int32)
+    q, k, v = O.qk_norm_rope_store(qkv, qw, kw, eps, cos, sin, k_cache, v_cache, slots, hq, hkv)
+
+    def bf(x):     # fp64 -> bf16 -> fp64
+        return float(torch.tensor(x, dtype=torch.float64).float().to(torch.bfloat16))
+
+    def front(row, w, t):
+        ms = sum(float(a) ** 2 for a in row) / d
+        normed = [bf(bf(float(a) / math.sqrt(ms + eps)) * float(wi)) for a, wi in zip(row, w)]
+        out = [0.0] * d
+        for i in range(half):
+            c, s = float(cos[t, 0, i]), float(sin[t, 0, i])
+            out[i] = bf(normed[i] * c - normed[half + i] * s)
+            out[half + i] = bf(normed[half + i] * c + normed[i] * s)
+        return out
+
+    tol = 2 ** -6
+    for t in range(T):
+        for h in range(hq):
+            want = front(qkv[t, h * d:(h + 1) * d].tolist(), qw.tolist(), t)
+            assert max(abs(a - b) for a, b in zip(q[t, h].double().tolist(), want)) <= tol * max(1.0, max(map(abs, want)))
+        want = front(qkv[t, hq * d:(hq + 1) * d].tolist(), kw.tolist(), t)
+        assert max(abs(a - b) for a, b in zip(k[t, 0].double().tolist(), want)) <= tol * max(1.0, max(map(abs, want)))
+    assert_bit_exact(v.reshape(T, d), qkv[:, (hq + hkv) * d:], "v is the raw slice of qkv")
+    kc, vc = k_cache.view(-1, d), v_cache.view(-1, d)
+    for t, s in enumerate(slots.tolist()):
+        if s >= 0:
+            assert_bit_exact(kc[s], k[t, 0], "rotated k in its slot")
+            assert_bit_exact(vc[s], v[t, 0], "raw v in its slot")
+    untouched = [i for i in range(8) if i not in (5, 2)]
+    assert (kc[untouched] == 7).all() and (vc[untouched] == 7).all()      # slot -1 skipped, nothing else written
