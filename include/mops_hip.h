@@ -28,7 +28,8 @@ extern "C" {
 #define MOPS_HIP_EUNSUPPORTED (-2) /* shape the kernels are not written for (head_dim, block size…)  */
 #define MOPS_HIP_EALIGN (-3)       /* pointer or stride breaks the 16-byte alignment the kernels need */
 #define MOPS_HIP_EWORKSPACE (-4)   /* workspace missing or smaller than mops_hip_*_workspace_bytes    */
-#define MOPS_HIP_ELAUNCH (-5)      /* hipLaunchKernel reported an error (see mops_hip_last_hip_error) */
+#define MOPS_HIP_ELAUNCH (-5)      /* a HIP call or launch reported an error (see mops_hip_last_hip_error) */
+#define MOPS_HIP_ETOOLARGE (-6)    /* problem exceeds the fixed scratch of an allocation-free entry point */
 
 /* ABI version of this header; bumped on any signature change. */
 int mops_hip_abi_version(void);
@@ -158,6 +159,28 @@ int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_strid
                                             float softmax_scale,
                                             void* workspace, int64_t workspace_bytes,
                                             int plan_mode, void* stream);
+
+/*
+ * Paged decode attention for callers that cannot allocate: code under HIP-graph capture, tight serving loops
+ * that hold no workspace, harnesses that forbid hipMalloc.  No counterpart in the reference.  Arguments and
+ * results are those of mops_hip_attn_paged_decode_bf16 (same kernels, bit-identical output) without the
+ * workspace pair: the split-context partials live in a fixed device array inside the library, one copy of
+ * MOPS_HIP_DECODE_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends.  The call allocates and frees
+ * nothing and does not synchronise.  A problem whose workspace (mops_hip_paged_decode_workspace_bytes) exceeds
+ * that size returns MOPS_HIP_ETOOLARGE and launches nothing; both benchmark shapes fit (4.3 MB at 256
+ * sequences x 16/8 heads, 8.5 MB at 512 x 32/8).  All calls on one GPU share that GPU's array: calls that
+ * overlap in time on one GPU (different streams, or threads) race; calls on one stream are ordered and safe.
+ * The first call on a GPU looks the array's device address up (hipGetSymbolAddress); make it outside capture.
+ */
+#define MOPS_HIP_DECODE_NOALLOC_SCRATCH_BYTES (16ll << 20)
+int mops_hip_attn_paged_decode_noalloc_bf16(const void* q, int64_t q_batch_stride,
+                                            const void* k_cache, const void* v_cache,
+                                            const int32_t* cache_seqlens,
+                                            const int32_t* block_table, int64_t block_table_row_stride,
+                                            void* out,
+                                            int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                            int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                            float softmax_scale, void* stream);
 
 /*
  * Varlen (packed, THD) causal prefill attention with grouped-query heads, with or without a cached prefix.

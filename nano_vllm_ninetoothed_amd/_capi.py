@@ -35,6 +35,9 @@ SIGNATURES = {
                                                 c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                 c_int64, c_int64, c_int64, c_float, c_void_p, c_int64,
                                                 c_int, c_void_p]),
+    "mops_hip_attn_paged_decode_noalloc_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                        c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                        c_int64, c_int64, c_int64, c_float, c_void_p]),
     "mops_hip_attn_varlen_causal_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                                  c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64,
                                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
@@ -52,7 +55,7 @@ SIGNATURES = {
     "mops_hip_linear_tune": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
 }
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib = None
 
@@ -98,6 +101,6 @@ def check(func: str, status: int) -> None:
     if status != 0:
         lib = load()
         text = lib.mops_hip_status_string(status).decode()
-        if status == -5:
+        if status == -5:  # MOPS_HIP_ELAUNCH
             text += f" (hipError {lib.mops_hip_last_hip_error()})"
         raise MopsHipError(func, status, text)

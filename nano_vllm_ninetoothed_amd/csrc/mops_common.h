@@ -61,5 +61,7 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // Records the launch error (if any) for mops_hip_last_hip_error and maps it to a status.
 int finish_launch();
+// Records a failed HIP runtime call the same way; returns MOPS_HIP_ELAUNCH.
+int record_hip_error(hipError_t e);
 
 }  // namespace mops

@@ -32,6 +32,7 @@
 //   moves between lanes.
 #include "mops_common.h"
 #include <stdlib.h>
+#include <mutex>
 
 namespace mops {
 
@@ -640,6 +641,32 @@ static int launch_paged_decode(const void* q, int64_t q_batch_stride,
   return finish_launch();
 }
 
+// Scratch of the allocation-free entry point: one copy per GPU, held until the process ends.  In host code
+// this name is only a handle for hipGetSymbolAddress; the device address it yields is what the kernels get.
+constexpr int64_t kStaticScratchBytes = MOPS_HIP_DECODE_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];   // device address of `scratch` on each GPU, looked up once
+static std::mutex g_scratch_mutex;
+
+// Device address of this GPU's copy of `scratch` (nullptr and a status on failure).
+static int static_scratch(void** ptr) {
+  *ptr = nullptr;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return record_hip_error(e != hipSuccess ? e : hipErrorInvalidDevice);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !addr) return record_hip_error(e != hipSuccess ? e : hipErrorInvalidSymbol);
+    g_scratch_ptr[dev] = addr;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return MOPS_HIP_OK;
+}
+
 }  // namespace mops
 
 extern "C" int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_batch_stride,
@@ -655,6 +682,30 @@ extern "C" int mops_hip_attn_paged_decode_planned_bf16(const void* q, int64_t q_
   return mops::launch_paged_decode(q, q_batch_stride, k_cache, v_cache, cache_seqlens, block_table, block_table_row_stride,
                                    out, batch, hq, hkv, head_dim, block_size, num_blocks, max_blocks_per_seq, softmax_scale,
                                    workspace, workspace_bytes, plan_mode, stream);
+}
+
+extern "C" int mops_hip_attn_paged_decode_noalloc_bf16(const void* q, int64_t q_batch_stride,
+                                                       const void* k_cache, const void* v_cache,
+                                                       const int32_t* cache_seqlens,
+                                                       const int32_t* block_table, int64_t block_table_row_stride,
+                                                       void* out,
+                                                       int64_t batch, int64_t hq, int64_t hkv, int64_t head_dim,
+                                                       int64_t block_size, int64_t num_blocks, int64_t max_blocks_per_seq,
+                                                       float softmax_scale, void* stream) {
+  using namespace mops;
+  if (batch <= 0 || hq <= 0 || hkv <= 0) {
+    // let the shared validation name the problem (or accept the empty batch); no scratch is needed for either
+    return launch_paged_decode(q, q_batch_stride, k_cache, v_cache, cache_seqlens, block_table, block_table_row_stride, out,
+                               batch, hq, hkv, head_dim, block_size, num_blocks, max_blocks_per_seq, softmax_scale,
+                               nullptr, 0, MOPS_HIP_DECODE_PLAN_AND_ATTEND, stream);
+  }
+  if (workspace_layout(batch, hq, choose_ncols(hkv)).total > kStaticScratchBytes) return MOPS_HIP_ETOOLARGE;
+  void* ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st != MOPS_HIP_OK) return st;
+  return launch_paged_decode(q, q_batch_stride, k_cache, v_cache, cache_seqlens, block_table, block_table_row_stride, out,
+                             batch, hq, hkv, head_dim, block_size, num_blocks, max_blocks_per_seq, softmax_scale,
+                             ws, kStaticScratchBytes, MOPS_HIP_DECODE_PLAN_AND_ATTEND, stream);
 }
 
 extern "C" int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
