@@ -12,6 +12,9 @@ A step is one flash_attn_with_kvcache call over the whole batch, KV cache reside
   copy = a plain 1 GiB device-to-device tensor copy (not a mops op): the known-size kernel against which
          the FETCH_SIZE / WRITE_SIZE counters of a profile are calibrated.
 
+The default line also carries an `e2e` block: the cfg5 workload's output tok/s with the decode step replayed from
+HIP graphs, once reading every step's tokens back (as the reference's loop does) and once pipelined (--no-e2e skips it).
+
 Prints ONE JSON line on stdout.  `roofline` is computed from HIP-event time of the op on its launch
 stream; `cpu_baseline` times the CPU restatement of the reference's torch backend (oracle/) on a
 bounded sample of the same workload on this machine's host cores.
@@ -26,6 +29,9 @@ import time
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the default workload, calibrated against a 1 GiB copy
+DECODE_TRAFFIC_BYTES = 2497.6e6
+DECODE_TRAFFIC_SOURCE = "profiles/hbm_traffic_decode_prefill.txt (rocprofv3 --pmc, not measured by this run)"
 
 
 def parse_args():
@@ -39,43 +45,72 @@ def parse_args():
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true", help="default op only: skip the end-to-end block of the line (profiling runs)")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
 
 
-def run_e2e(args, torch, dev, mops):
-    """Workload of the reference's bench.py:9-28 on the engine counterpart, hip backend; plus a reduced
-    run of the same engine on the CPU-restated torch backend (on the GPU) as the comparison baseline."""
+def e2e_workload(n):
+    """Prompts and output lengths of the reference's bench.py:9-28 (random.seed(0), token ids 0..10000)."""
     import random
-    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
     random.seed(0)
-    n = args.e2e_seqs
     prompts = [[random.randint(0, 10000) for _ in range(random.randint(100, 1024))] for _ in range(n)]
     max_tokens = [random.randint(100, 1024) for _ in range(n)]
+    return prompts, max_tokens
+
+
+def e2e_modes(args, torch, modes):
+    """Runs the e2e workload once per mode on one engine (random-init Qwen3-0.6B architecture, hip backend).
+    Modes: "pipelined" (decode step replayed from HIP graphs, sampled tokens kept on the device and read back once
+    at the end), "stepwise" (graphs, every step's tokens read back before the next step is scheduled, as
+    nanovllm/engine/model_runner.py:212 does), "eager" (no graphs, per-step readback: the reference's
+    enforce_eager=True setting, bench.py:15).  Returns {mode: {...}} in the order given."""
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    n = args.e2e_seqs
+    prompts, max_tokens = e2e_workload(n)
+    total = sum(max_tokens)
     eng = Engine(Qwen3Shape(), backend="hip", num_blocks=max(64, n * 10), seed=args.seed)
     eng.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 8)                 # warm-up, as the reference does
-    eng.pipelined = not args.e2e_stepwise
-    if not args.e2e_eager:
-        eng.capture_decode_graphs(max_bs=min(512, max(16, (n + 15) // 16 * 16)), max_model_len=4096)
-    _, st = eng.generate(prompts, max_tokens, temperature=0.6)
-    total = sum(max_tokens)
+    res = {}
+    for mode in sorted(modes, key=lambda m: m != "eager"):       # eager first: it must run before graphs exist
+        if mode != "eager" and not eng.graphs:
+            eng.capture_decode_graphs(max_bs=min(512, max(16, (n + 15) // 16 * 16)), max_model_len=4096)
+        eng.pipelined = mode == "pipelined"
+        _, st = eng.generate(prompts, max_tokens, temperature=0.6)
+        assert not eng.running and not eng.waiting and len(eng.free_blocks) == eng.num_blocks
+        res[mode] = {"mode": mode, "tok_per_s": round(total / st["total_s"], 1), "output_tokens": total,
+                     "seconds": round(st["total_s"], 3), "prompt_tokens": sum(len(p) for p in prompts),
+                     "prefill_steps": st["prefill_steps"], "decode_steps": st["decode_steps"],
+                     "prefill_tok_per_s": round(st["prefill_tokens"] / max(st["prefill_s"], 1e-9), 1),
+                     "decode_tok_per_s": round(st["decode_tokens"] / max(st["decode_s"], 1e-9), 1)}
+    del eng
+    torch.cuda.empty_cache()
+    return {m: res[m] for m in modes}
+
+
+E2E_WORKLOAD_TEXT = ("cfg5 end-to-end generate, random-init Qwen3-0.6B architecture (28 layers, hidden 1024, 16/8 heads, "
+                     "vocab 151936, tied embeddings), mops hip backend, engine counterpart of the reference's bench.py:9-28")
+
+
+def run_e2e(args, torch, dev, mops):
+    """`--op e2e`: the cfg5 workload as the line's own metric, plus a reduced run of the same engine on the
+    CPU-restated torch backend (on the GPU) as the comparison baseline."""
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    mode = "eager" if args.e2e_eager else ("stepwise" if args.e2e_stepwise else "pipelined")
+    r = e2e_modes(args, torch, [mode])[mode]
+    n = args.e2e_seqs
+    prompts, _ = e2e_workload(n)
+    steps = r["prefill_steps"] + r["decode_steps"]
     out = {
-        "metric": "e2e_output_tok_per_s", "value": round(total / st["total_s"], 2), "unit": "tok/s", "n_gpus": 1,
-        "steps": st["prefill_steps"] + st["decode_steps"], "warmup": 1,
-        "ms_per_step": round(st["total_s"] * 1e3 / (st["prefill_steps"] + st["decode_steps"]), 4),
+        "metric": "e2e_output_tok_per_s", "value": r["tok_per_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": steps, "warmup": 1, "ms_per_step": round(r["seconds"] * 1e3 / steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "cfg5 end-to-end generate, random-init Qwen3-0.6B architecture, mops hip backend, decode step "
-                               + ("eager" if args.e2e_eager else "replayed from HIP graphs")
-                               + ("" if args.e2e_eager or args.e2e_stepwise else ", tokens read back once at the end"),
+        "config": {"workload": E2E_WORKLOAD_TEXT + ", mode " + mode,
                    "prompts": n, "prompt_len": "uniform[100,1024]", "max_tokens": "uniform[100,1024]", "temperature": 0.6,
-                   "output_tokens": total, "prompt_tokens": sum(len(p) for p in prompts)},
-        "breakdown": {"seconds": round(st["total_s"], 3), "prefill_steps": st["prefill_steps"], "decode_steps": st["decode_steps"],
-                      "prefill_tok_per_s": round(st["prefill_tokens"] / max(st["prefill_s"], 1e-9), 1),
-                      "decode_tok_per_s": round(st["decode_tokens"] / max(st["decode_s"], 1e-9), 1)},
+                   "output_tokens": r["output_tokens"], "prompt_tokens": r["prompt_tokens"]},
+        "breakdown": r,
     }
     if not args.no_cpu_baseline:
-        del eng
-        torch.cuda.empty_cache()
         import oracle.mops_torch  # noqa: F401  comparison backend only
         m, outlen = 16, 16
         res = {}
@@ -127,6 +162,7 @@ def main():
 
     cpu_fn = None      # () -> (seconds, description, units_done)  on a bounded sample
     measured_traffic = None
+    traffic_source = None
 
     if args.op == "e2e":
         run_e2e(args, torch, dev, mops)
@@ -169,9 +205,13 @@ def main():
                   "block_size": W.BLOCK_SIZE, "context": f"uniform[{lo},{hi}] seed {args.seed}",
                   "context_tokens": sum(ctx), "kv_buffers_rotated": n_copies}
         kernel_name = "paged_decode_kernel (+ paged_decode_plan_kernel, paged_decode_combine_kernel)"
-        # HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this exact
-        # workload (profiles/hbm_traffic_decode_prefill.txt); only valid for the default seed
-        measured_traffic = 2497.6e6 if (args.op == "decode" and args.seed == 0) else None
+        # HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this exact workload;
+        # a figure copied from that profile, not measured by this run: only given for the default seed and
+        # launch shape, with its source next to it
+        tuned = any(os.environ.get(v) for v in ("MOPS_HIP_DECODE_HPW", "MOPS_HIP_DECODE_NCOLS", "MOPS_HIP_DECODE_MIN_PER_COL"))
+        if args.op == "decode" and args.seed == 0 and not tuned:
+            measured_traffic = DECODE_TRAFFIC_BYTES
+            traffic_source = DECODE_TRAFFIC_SOURCE
 
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401
@@ -378,7 +418,8 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic", "config": config,
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": runit,
-                     "frac": round(achieved / peak, 4), "traffic": measured_traffic, "kernel": kernel_name,
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic, "traffic_source": traffic_source,
+                     "kernel": kernel_name,
                      "algorithmic_work_per_launch": work, "event_ms_per_launch": round(ev_ms, 5),
                      "event_ms_min": round(min(per_step_ms), 5)},
     }
@@ -388,6 +429,14 @@ def main():
         cval = units / secs / (1e9 if bound == "hbm" else 1e12)
         out["cpu_baseline"] = {"value": round(cval, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
                                "sample": sample, "seconds": round(secs, 4)}
+    if args.op == "decode" and not args.no_e2e:
+        # second half of the headline metric: end-to-end output tok/s of the cfg5 workload, in the two graph modes
+        step = op = caches = q = None
+        torch.cuda.empty_cache()
+        r = e2e_modes(args, torch, ["stepwise", "pipelined"])
+        out["e2e"] = {"metric": "e2e_output_tok_per_s", "unit": "tok/s", "workload": E2E_WORKLOAD_TEXT,
+                      "prompts": args.e2e_seqs, "prompt_len": "uniform[100,1024]", "max_tokens": "uniform[100,1024]",
+                      "temperature": 0.6, "runs": [r["stepwise"], r["pipelined"]]}
     print(json.dumps(out))
 
 

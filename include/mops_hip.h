@@ -196,8 +196,9 @@ int mops_hip_attn_paged_decode_noalloc_bf16(const void* q, int64_t q_batch_strid
  *   sequence s is row cu_k[s] + j; cu_seqlens_k may be NULL (then it equals cu_seqlens_q).
  * block_table != NULL: k/v are the contiguous paged caches [num_blocks, block_size, hkv, 128] and key j of
  *   sequence s is cache[block_table[s, j/block_size], j%block_size] (row stride block_table_row_stride,
- *   at least max_blocks_per_seq columns; entries beyond the sequence's keys are never read; block_size
- *   must be a multiple of 64); k/v token strides are ignored.
+ *   at least max_blocks_per_seq columns; entries beyond the sequence's keys are never read; an entry
+ *   outside [0, num_blocks) inside the used range is treated as an empty block, i.e. its keys get no weight,
+ *   the rule of the decode entry points; block_size must be a multiple of 64); k/v token strides are ignored.
  * cu_seqlens_*: int32 [batch+1], non-decreasing, starting at 0.  max_seqlen_q bounds every query length
  * and only sizes the launch.  Sequences of length 0 are allowed.
  */
@@ -238,7 +239,10 @@ int mops_hip_apply_rotary_emb(const void* x, int64_t x_token_stride, int64_t x_h
 /*
  * sampler_forward — out[r] = argmax(softmax(logits[r, :] / temperature[r])) for positive temperatures, i.e.
  * the index of the row's largest logit (first index on ties).  The temperatures do not change the result
- * and are not passed.  Replaces: mops/torch/ops.py:37-43 (greedy: the Gumbel line is commented out),
+ * and are not passed.  A row holding a NaN or +inf logit, or only -inf, gives 0: the library softmax turns such a row
+ * into NaNs and its argmax of an all-NaN row is 0.  Not reproduced: temperatures <= 0 (the library expression yields
+ * inf/NaN garbage) and logits so close to zero that they collide after the fp32 division and exponential
+ * (|logit| / T below ~1e-5, where every candidate is equally tiny).  Replaces: mops/torch/ops.py:37-43 (greedy: the Gumbel line is commented out),
  * mops/ninetoothed/sampler_forward.py:9-94; called at nanovllm/layers/sampler.py:12.
  * logits: [rows, n] bf16 with row stride in elements (% 8 == 0); out: int64 [rows].
  */

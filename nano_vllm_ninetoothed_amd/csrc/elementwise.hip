@@ -141,9 +141,12 @@ __global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16
                                                                    int64_t* __restrict__ out, int n) {
   __shared__ float best_v[kArgmaxThreads / kWave];
   __shared__ int best_i[kArgmaxThreads / kWave];
+  __shared__ int spoiled_w[kArgmaxThreads / kWave];
   const uint16_t* row = logits + (int64_t)blockIdx.x * row_stride;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
+  // A NaN or +inf logit turns the whole softmax row into NaN, and the library's argmax of an all-NaN row is 0.
+  bool spoiled = false;
   const int pieces = n >> 3;
   for (int pc = threadIdx.x; pc < pieces; pc += kArgmaxThreads) {
     const u32x4 w = load16_stream(row + (pc << 3));
@@ -151,15 +154,17 @@ __global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16
     for (int e = 0; e < 4; ++e) {
       const float lo = bf16lo_to_f32(w[e]), hi = bf16hi_to_f32(w[e]);
       const int i0 = (pc << 3) + 2 * e;
+      spoiled |= !(lo < INFINITY) || !(hi < INFINITY);
       if (lo > bv) { bv = lo; bi = i0; }        // strictly greater: within a lane indices only grow
       if (hi > bv) { bv = hi; bi = i0 + 1; }
     }
   }
   for (int i = (pieces << 3) + threadIdx.x; i < n; i += kArgmaxThreads) {  // tail when n % 8 != 0
     const float x = bf16lo_to_f32(row[i]);
+    spoiled |= !(x < INFINITY);
     if (x > bv) { bv = x; bi = i; }
   }
-  // NaN never compares greater; a row of NaNs yields index 0 like an all -inf row would
+  // an all -inf row is all NaN after the softmax as well: bi stays unset and becomes 0 below
 #pragma unroll
   for (int off = kWave / 2; off >= 1; off >>= 1) {
     const float ov = __shfl_xor(bv, off, kWave);
@@ -170,11 +175,15 @@ __global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16
     best_v[threadIdx.x / kWave] = bv;
     best_i[threadIdx.x / kWave] = bi;
   }
+  const bool wave_spoiled = __any(spoiled);
+  if ((threadIdx.x & (kWave - 1)) == 0) spoiled_w[threadIdx.x / kWave] = wave_spoiled;
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < kArgmaxThreads / kWave; ++w)
       if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
-    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    bool any_spoiled = false;
+    for (int w = 0; w < kArgmaxThreads / kWave; ++w) any_spoiled |= spoiled_w[w] != 0;
+    out[blockIdx.x] = (bi == 0x7fffffff || any_spoiled) ? 0 : bi;
   }
 }
 

@@ -276,7 +276,9 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   const uint16_t* kptr = p.k + (int64_t)(kbegin + ld_row) * p.k_ts + col;
   const uint16_t* vptr = p.v + (int64_t)(kbegin + ld_row) * p.v_ts + col;
   const int32_t* table = paged ? p.block_table + (int64_t)b * p.block_table_row_stride : nullptr;
-  auto load_tile = [&](const uint16_t* base, const uint16_t* cache, int64_t ts, int tile, u32x4 (&r)[4]) {
+  // returns false when the tile's cache block does not exist (table entry outside [0, num_blocks)): the tile
+  // then reads as zeros and the caller masks all of its keys
+  auto load_tile = [&](const uint16_t* base, const uint16_t* cache, int64_t ts, int tile, u32x4 (&r)[4]) -> bool {
     const uint16_t* src;
     bool tile_ok = true;
     if (paged) {  // a 64-token tile lies inside one cache block (block_size is a multiple of 64)
@@ -300,6 +302,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         r[i] = x;
       }
     }
+    return tile_ok;
   };
   const int st_k = ld_row * kPKStride + (ld_slice << 4);
   const int st_v = ld_row * kPVStride + (ld_slice << 4);
@@ -312,8 +315,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds_v + buf * kPVTile + st_v + 16 * i * kPVStride) = r[i];
   };
   // wave-uniform base address of a tile's first token; true when the whole tile can be loaded unconditionally
-  auto tile_base = [&](const uint16_t* packed, int64_t ts, int tile, const char*& base) -> bool {
-    bool tile_ok = true;
+  auto tile_base = [&](const uint16_t* packed, int64_t ts, int tile, const char*& base, bool& tile_ok) -> bool {
+    tile_ok = true;
     if (paged) {
       const int t0 = tile * kPBN;
       const int blk = table[t0 / p.block_size];
@@ -352,7 +355,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   //   block A: S^T = K . Q^T, the eight global loads of the next tile ride in its slots
   //   block B: row max, rescale factor, the first eight exponentials
   //   block C: O^T += V^T . P^T, the remaining exponentials and the eight LDS stores of the next tile ride in its slots
-  auto tile_compute = [&](int tile, const char* kbase, const char* vbase, auto move, auto masked) {
+  // `horizon`: last key (sequence-relative) this lane's row may see; only read on the masked variant.
+  auto tile_compute = [&](int tile, const char* kbase, const char* vbase, auto move, auto masked, int horizon) {
     const int buf = tile & 1;
     f32x16 s[2];
     {
@@ -387,7 +391,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
-          s[tt][r] = key <= my_row + shift ? s[tt][r] : -INFINITY;
+          s[tt][r] = key <= horizon ? s[tt][r] : -INFINITY;
         }
     }
     // A wave issues in order and a dependent VALU instruction waits ~20 cycles for its operand, so the
@@ -476,7 +480,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 
   // ---- tile loop.  The next tile travels HBM -> registers during block A and registers -> the other LDS
   //      buffer during block C; that buffer was last read before this tile's barrier.
-  load_tile(kptr, p.k, p.k_ts, 0, kreg);
+  bool tile_exists = load_tile(kptr, p.k, p.k_ts, 0, kreg);   // the tile about to be computed has a cache block
   load_tile(vptr, p.v, p.v_ts, 0, vreg);
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
@@ -497,8 +501,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const int64_t kstep = (int64_t)kPBN * p.k_ts * 2, vstep = (int64_t)kPBN * p.v_ts * 2;
     for (; tile < n_fast; ++tile) {
       lds_barrier();
-      if (tile < unmasked) tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{});
-      else tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{});
+      if (tile < unmasked) tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{}, 0);
+      else tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{}, my_row + shift);
       kbase += kstep;
       vbase += vstep;
     }
@@ -508,31 +512,34 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const bool have_next = tile + 1 < ntiles;
     const char* kbase = nullptr;
     const char* vbase = nullptr;
-    bool sliced = false;
+    bool sliced = false, next_exists = true;
     if (have_next && tile < my_tiles) {
-      const bool k_whole = tile_base(p.k, p.k_ts, tile + 1, kbase);
-      const bool v_whole = tile_base(p.v, p.v_ts, tile + 1, vbase);
+      const bool k_whole = tile_base(p.k, p.k_ts, tile + 1, kbase, next_exists);
+      const bool v_whole = tile_base(p.v, p.v_ts, tile + 1, vbase, next_exists);
       sliced = k_whole && v_whole;
     }
-    // the mask is only needed where the tile holds a key beyond the first row's horizon
-    const bool masked = tile * kPBN + kPBN - 1 > wave_row0 + shift;
+    // the mask is only needed where the tile holds a key beyond the first row's horizon; a tile whose cache
+    // block does not exist (it was loaded as zeros) is masked as a whole: its keys get no weight, as in decode
+    const bool masked = tile * kPBN + kPBN - 1 > wave_row0 + shift || !tile_exists;
+    const int horizon = tile_exists ? my_row + shift : -1;
     if (sliced) {
-      if (masked) tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{});
-      else tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{});
+      if (masked) tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{}, horizon);
+      else tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{}, 0);
     } else {
       if (have_next) {
-        load_tile(kptr, p.k, p.k_ts, tile + 1, kreg);
+        next_exists = load_tile(kptr, p.k, p.k_ts, tile + 1, kreg);
         load_tile(vptr, p.v, p.v_ts, tile + 1, vreg);
       }
       if (tile < my_tiles) {
-        if (masked) tile_compute(tile, kbase, vbase, std::false_type{}, std::true_type{});
-        else tile_compute(tile, kbase, vbase, std::false_type{}, std::false_type{});
+        if (masked) tile_compute(tile, kbase, vbase, std::false_type{}, std::true_type{}, horizon);
+        else tile_compute(tile, kbase, vbase, std::false_type{}, std::false_type{}, 0);
       }
       if (have_next) {
         store_k((tile + 1) & 1, kreg);
         store_v((tile + 1) & 1, vreg);
       }
     }
+    tile_exists = next_exists;
   }
 
   // ---- epilogue.  A lane holds 8-byte pieces of its own row, which would make every store instruction

@@ -386,8 +386,10 @@ def siluAndMul(x: torch.Tensor, y: torch.Tensor):
 @register_hip_op
 def sampler_forward(logits: torch.Tensor, temperatures: torch.Tensor):
     """argmax(softmax(logits / T)) per row -> int64 [B] (mops/torch/ops.py:37-43; the reference samples
-    greedily).  For positive temperatures that is the index of the largest logit, computed in one pass
-    over the bf16 logits; other dtypes and layouts take the library expression."""
+    greedily).  For positive temperatures that is the index of the largest logit (the first on ties), computed in
+    one pass over the bf16 logits; a row with a NaN or +inf logit gives 0, as the library expression does.
+    Assumes temperatures > 0: with T <= 0 the reference's expression produces inf/NaN garbage, which is not
+    reproduced.  Other dtypes and layouts take the library expression."""
     if logits.is_cuda and logits.dtype == torch.bfloat16 and logits.dim() == 2 and logits.stride(1) == 1 \
             and logits.stride(0) % 8 == 0 and logits.data_ptr() % 16 == 0:
         rows, n = logits.shape

@@ -69,8 +69,11 @@ def assert_rms_parity(got: torch.Tensor, normed_ref: torch.Tensor, weight: torch
     """RMSNorm has two bf16 roundings: bf16(x * rstd), then bf16(that * w).  The row statistic is an fp32
     sum whose last bit depends on summation order, which can move the FIRST rounding by one bf16 step.
     Accepted: the output equals, bit for bit, what the reference's second stage produces from a
-    normalised value at most 1 bf16 ulp from the reference's (normed_ref); and at least 99.9 % of the
-    elements equal the reference output exactly."""
+    normalised value at most 1 bf16 ulp from the reference's (normed_ref); at least 99.9 % of the
+    elements equal the reference output exactly; and, measured on the final output, no element is more than
+    2 bf16 ulp from the reference and at most one in 100 000 is more than 1 ulp away (a one-step move of the
+    first rounding, multiplied by a weight, can land two steps away after the second rounding).  The
+    measured distances are printed (pytest -s) and returned."""
     got = got.cpu()
     assert got.shape == want.shape and got.dtype == torch.bfloat16
     assert torch.isfinite(got.float()).all(), f"{what}: non-finite"
@@ -85,3 +88,12 @@ def assert_rms_parity(got: torch.Tensor, normed_ref: torch.Tensor, weight: torch
     assert bad == 0, f"{what}: {bad} elements are not reachable from a normalised value within 1 bf16 ulp"
     exact = (gb == want.contiguous().view(torch.int16)).float().mean().item()
     assert exact >= 0.999, f"{what}: only {exact:.5f} of the elements equal the reference bit for bit"
+    dist = ulp_distance_bf16(got, want)
+    worst = int(dist.max()) if dist.numel() else 0
+    beyond_one = int((dist > 1).sum())
+    allowed = -(-dist.numel() // 100000)    # ceil(numel / 1e5)
+    print(f"[rms parity] {what}: {dist.numel()} elements, {exact * 100:.4f} % bit-equal, max {worst} bf16 ulp, "
+          f"{beyond_one} beyond 1 ulp (allowed {allowed})")
+    assert worst <= 2, f"{what}: an output is {worst} bf16 ulp from the reference (allowed 2)"
+    assert beyond_one <= allowed, f"{what}: {beyond_one} outputs are more than 1 bf16 ulp from the reference (allowed {allowed})"
+    return {"elements": dist.numel(), "bit_equal": exact, "max_ulp": worst, "beyond_one_ulp": beyond_one}

@@ -71,6 +71,18 @@ def test_embedding_matches_oracle(gpu, ops, n_ids, vocab, hidden, dtype):
     assert_bit_exact(got, torch.nn.functional.embedding(d["ids"].long(), d["weight"]), "embedding vs F.embedding")
 
 
+def test_embedding_full_size_8b_table(gpu, ops):
+    """The Qwen3-8B-shaped case at its exact size: 512 int32 ids uniform over a bf16 [151936, 4096] table ~N(0, 0.02)
+    (1.24 GB), bit-exact against weight[ids] (nanovllm/layers/embed_head.py:41)."""
+    hip, ref = ops("embedding")
+    d = W.embedding_inputs(512, 151936, 4096, seed=0, id_dtype=torch.int32)
+    assert d["ids"].dtype == torch.int32 and d["weight"].shape == (151936, 4096)
+    got = hip(d["ids"].to(gpu), d["weight"].to(gpu))
+    assert got.shape == (512, 4096)
+    assert_bit_exact(got, d["weight"][d["ids"].long()], "embedding, 151936 x 4096 table")
+    assert_bit_exact(got, ref(d["ids"], d["weight"]), "embedding vs oracle")
+
+
 def test_embedding_2d_ids_and_empty(gpu, ops):
     hip, ref = ops("embedding")
     d = W.embedding_inputs(48, 3000, 1024, seed=9, id_dtype=torch.int64)

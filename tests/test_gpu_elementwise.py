@@ -70,6 +70,25 @@ def test_sampler_matches_oracle(gpu, ops, rows, vocab):
     assert int(got[0]) == 3
 
 
+def test_sampler_on_rows_the_softmax_turns_into_nans(gpu, ops):
+    """A NaN or +inf logit, or a row of -inf, makes softmax(logits / T) all NaN, and the library's argmax of an
+    all-NaN row is 0; the kernel answers the same.  Rows around them are unaffected."""
+    hip, ref = ops("sampler_forward")
+    g = torch.Generator().manual_seed(77)
+    logits = (torch.randn((6, 4096), generator=g) * 3).to(torch.bfloat16)
+    logits[0, 100] = float("nan")
+    logits[1, 4095] = float("inf")
+    logits[2, :] = float("-inf")
+    logits[3, 7] = float("nan"); logits[3, 9] = 80.0
+    logits[4, 1234] = 70.0                           # an ordinary row
+    logits[5, 17] = float("-inf")                    # -inf entries alone are harmless
+    temps = torch.full((6,), 0.6)
+    want = ref(logits, temps)
+    got = hip(logits.to(gpu), temps.to(gpu)).cpu()
+    assert torch.equal(got, want), (got.tolist(), want.tolist())
+    assert got[:4].tolist() == [0, 0, 0, 0] and int(got[4]) == 1234
+
+
 @pytest.mark.parametrize("tokens,hq,hkv,need_k", [(1, 16, 8, True), (5, 16, 8, False), (300, 16, 8, True), (64, 32, 8, False), (33, 8, 1, True)])
 def test_fused_qk_norm_rope_store_equals_the_separate_ops(gpu, tokens, hq, hkv, need_k):
     """qk_norm_rope_store against the sequence it replaces, both through the hip backend: bit-identical q, k

@@ -151,3 +151,29 @@ def test_shipped_gemm_solution_table_is_applied(gpu):
     version; if either differs the loader pins nothing and the engine silently runs on the heuristic's picks."""
     from nano_vllm_ninetoothed_amd.mops.hip.ops import load_linear_solutions
     assert load_linear_solutions() > 0
+
+
+def test_full_size_engine_pipelined_equals_stepwise(gpu):
+    """The end-to-end configuration at its real shape: random-init Qwen3-0.6B architecture (28 layers, vocab
+    151936), 64 prompts of 100..1024 random tokens, graph buckets up to 256 sequences.  Pipelined generation must
+    give the stepwise loop's tokens; every sequence gets exactly its max_tokens and all cache blocks come back."""
+    import random
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    shape = Qwen3Shape()
+    assert (shape.num_layers, shape.vocab, shape.hidden, shape.num_heads, shape.num_kv_heads) == (28, 151936, 1024, 16, 8)
+    random.seed(0)
+    prompts = [[random.randint(0, 10000) for _ in range(random.randint(100, 1024))] for _ in range(64)]
+    max_tokens = [random.randint(8, 48) for _ in range(64)]
+    eng = Engine(shape, backend="hip", num_blocks=64 * 5, seed=0, device=str(gpu))
+    eng.capture_decode_graphs(max_bs=256, max_model_len=4096)
+    assert eng.graph_bs[-1] == 256
+    runs = []
+    for pipelined in (True, False):
+        eng.pipelined = pipelined
+        outs, stats = eng.generate(prompts, max_tokens)
+        assert [len(o) for o in outs] == max_tokens
+        assert all(0 <= t < shape.vocab for o in outs for t in o)
+        assert len(eng.free_blocks) == eng.num_blocks and not eng.running and not eng.waiting
+        assert stats["decode_tokens"] + 64 == sum(max_tokens)       # the first token of a sequence comes from its prefill
+        runs.append(outs)
+    assert runs[0] == runs[1], "pipelined and stepwise generation disagree"

@@ -139,6 +139,32 @@ def test_prefill_with_cached_prefix_matches_oracle(gpu, ops, new, prefix, hq, hk
     assert_bit_exact(got_packed, got, "packed keys with cu_seqlens_k vs paged keys")
 
 
+def test_prefix_prefill_treats_a_missing_block_as_empty(gpu, ops):
+    """A block_table entry outside [0, num_blocks) inside the used range: the keys of that block get no weight (the
+    rule paged decode follows for the same metadata), instead of entering the softmax with score 0."""
+    hip, _ = ops("flash_attn_varlen_func")
+    d = W.prefix_prefill_inputs([100, 300], [512, 300], seed=12)
+    table = d["block_table"].clone()
+    table[0, 1] = -1                      # keys 256..511 of sequence 0 (inside its cached prefix)
+    table[1, 0] = d["k_cache"].shape[0]   # keys 0..255 of sequence 1: one past the last block
+    g = W.to_device(d, gpu)
+    got = hip(g["q"], g["k_cache"], g["v_cache"], max_seqlen_q=d["max_seqlen_q"], cu_seqlens_q=g["cu_seqlens_q"],
+              max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=g["cu_seqlens_k"], softmax_scale=d["scale"], causal=True,
+              block_table=table.to(gpu))
+    cq, ck = d["cu_seqlens_q"].tolist(), d["cu_seqlens_k"].tolist()
+    want = torch.zeros_like(d["q"])
+    for s, dead in ((0, range(256, 512)), (1, range(0, 256))):
+        q = d["q"][cq[s]:cq[s + 1]].float().transpose(0, 1)                                    # [Hq, Lq, D]
+        k = d["k_all"][ck[s]:ck[s + 1]].float().transpose(0, 1).repeat_interleave(2, dim=0)  # [Hq, Lk, D]
+        v = d["v_all"][ck[s]:ck[s + 1]].float().transpose(0, 1).repeat_interleave(2, dim=0)
+        lq, lk = q.shape[1], k.shape[1]
+        scores = q @ k.transpose(1, 2) * d["scale"]
+        i, j = torch.arange(lq).unsqueeze(1), torch.arange(lk).unsqueeze(0)
+        hidden = (j > i + (lk - lq)) | torch.isin(j, torch.tensor(list(dead)))
+        want[cq[s]:cq[s + 1]] = (torch.softmax(scores.masked_fill(hidden, float("-inf")), -1) @ v).transpose(0, 1).to(torch.bfloat16)
+    assert_attention_close(got, want, "prefix prefill with two missing blocks")
+
+
 def test_prefill_is_bitwise_reproducible(gpu, ops):
     """The same launch repeated gives the same bits (plain, packed-with-prefix and paged inputs).  Guards the
     kernel's hand-placed instruction order: a VALU read of an MFMA result that comes too early returns
