@@ -69,6 +69,7 @@ constexpr int kPKStride = 272;      // bytes between K rows in LDS
 constexpr int kPVStride = 320;      // bytes between V rows in LDS
 constexpr int kPKTile = kPBN * kPKStride;   // 17408
 constexpr int kPVTile = kPBN * kPVStride;   // 20480
+constexpr float kLazyLog2 = 8.0f;    // the softmax reference moves when a row maximum outgrows it by this much (base-2 exponent)
 constexpr int kPCompactChunks = 4;  // the compact launch handles up to 64 * 4 sequences
 
 struct PrefillParams {
@@ -232,8 +233,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     kend = p.cu_seqlens_k[b + 1];
   }
   const int seq_len = min(seq_end, p.total_tokens) - seq_begin;   // query rows of this sequence
-  const int q0 = m * kPBM;
-  if (seq_begin < 0 || q0 >= seq_len) return;
+  // q tiles are aligned to the END of the sequence: tile m covers rows [q0, q0 + 128) with q0 = len - 128 * (tiles - m),
+  // so the partial tile is the first one (q0 < 0, rows below 0 do not exist), which looks at one or two K/V tiles, and
+  // not the last one, which looks at all of them: the rows a partial tile leaves idle cost almost nothing there.
+  const int seq_tiles = (seq_len + kPBM - 1) / kPBM;
+  if (seq_begin < 0 || seq_len <= 0 || m >= seq_tiles) return;
+  const int q0 = seq_len - (seq_tiles - m) * kPBM;
   // keys of this sequence: kv_len >= seq_len when a cached prefix precedes the new tokens; query row i
   // then sees keys 0 .. i + shift (bottom-right aligned causal mask)
   int kv_len = kend - kbegin;
@@ -258,7 +263,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   // ---- Q^T as B operand: lane (n, jj) holds Q[my_row][16*kb + 8*jj .. +8) for kb = 0..7
   bf16x8 qb[8];
   {
-    const bool row_ok = my_row < seq_len;
+    const bool row_ok = my_row >= 0 && my_row < seq_len;
     const uint16_t* qrow = p.q + (int64_t)(seq_begin + (row_ok ? my_row : 0)) * p.q_ts + (int64_t)h * kPD;
 #pragma unroll
     for (int kb = 0; kb < 8; ++kb) {
@@ -407,11 +412,20 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int c = 0; c < 4; ++c) mx[c] = max3(mx[c], s[c >> 1][8 * (c & 1) + 5], s[c >> 1][8 * (c & 1) + 6]);
     const float m01 = max3(mx[0], mx[1], s[0][7]), m23 = max3(mx[2], mx[3], s[0][15]);
     const float m_loc = half_swap_max(max3(m01, m23, fmaxf(s[1][7], s[1][15])));
-    const float m_new = fmaxf(m_run, m_loc);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    // The softmax reference m_run only moves when a row's maximum outgrows it by kLazyLog2 in the exponent's base-2
+    // units: probabilities then reach at most 2^kLazyLog2 (harmless in bf16 and in the fp32 sums, and the final
+    // division by the row sum is exact for any reference), and the 64 accumulator multiplies of a rescale, behind
+    // which nothing else can be issued, run on a row's first tile or two instead of on every other tile.
+    float alpha = 1.0f;
+    const bool grow = m_loc * p.scale_log2 > m_run * p.scale_log2 + kLazyLog2;   // -inf reference: any finite maximum
+    if (__any(grow)) {
+      const float m_new = grow ? m_loc : m_run;
+      const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_new_safe * p.scale_log2);
+      m_run = m_new;
+    }
+    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
     const float mc = m_safe * p.scale_log2;
-    const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - mc);
-    m_run = m_new;
     u32x4 pw[4];   // P^T as B operand for the four 16-token k blocks
     float ps0 = 0.f, ps1 = 0.f;
     float f0[16], f1[16];   // per element pair q = 0..15 (elements 2q, 2q+1 of this lane's 32 scores): stage values
@@ -567,7 +581,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int i = 0; i < 8; ++i) {
       const int row = row4 + 4 * i;
       const u32x4 w = *reinterpret_cast<const u32x4*>(stage + row * kOStride + 16 * piece);
-      if (wave_row0 + row < seq_len) *reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts) = w;
+      if (wave_row0 + row >= 0 && wave_row0 + row < seq_len) *reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts) = w;
     }
   }
 }
