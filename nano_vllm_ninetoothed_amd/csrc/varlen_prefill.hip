@@ -13,7 +13,7 @@
 // MFMA opens a slot, and what the wave issues while that MFMA runs is fixed by scheduling fences
 //   block A   S^T = K . Q^T           16 x v_mfma_f32_32x32x16_bf16 per wave; Q^T stays in registers as
 //                                      the B operand; the K operand reads run four MFMAs ahead of use;
-//                                      the eight global loads of the next tile ride in the slots
+//                                      the eight direct-to-LDS loads of the next tile ride in the slots
 //   block B   softmax head             each lane owns one q row, so the row max is register-local
 //                                      (four v_max3 chains) plus one half-wave swap
 //                                      (v_permlane32_swap); rescale factor; the scale is folded into
@@ -22,8 +22,8 @@
 //   block C   O^T += V^T . P^T         16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
 //                                      already the B-operand layout, V^T comes out of LDS through
 //                                      ds_read_b64_tr_b16 four MFMAs ahead; the exponent pipeline
-//                                      (scale, exp2, sum and pack), skewed one slot per stage, and the
-//                                      eight LDS stores of the next tile ride in the slots
+//                                      (scale, exp2, sum and pack), skewed one slot per stage, rides in
+//                                      the slots
 // In the steady part of the tile loop the per-tile bookkeeping is two pointer increments.
 //
 // What was measured on this part and shaped the kernel:
@@ -52,9 +52,12 @@
 //     ds_read_b128, but replacing it by plain reads of a pre-transposed tile changed the run time by
 //     2 %: the LDS pipe is not what bounds this shape.
 //
-// LDS rows are padded instead of swizzled (K rows 272 B apart, V rows 320 B apart): the K operand read
-// (16 consecutive rows, one 16-byte piece) and the transposing V read (4 rows x 4 pieces) each cover
-// all 64 banks once, and every address a lane needs is one base register plus an immediate.
+// K/V tiles travel HBM -> LDS directly (global_load_lds_dwordx4, no stop in registers), so LDS rows are unpadded
+// (256 B, the two double-buffered tile pairs fill exactly 64 KiB) and bank conflicts are avoided by a swizzle applied
+// on the global side of the load: 16-byte position pos of K row r holds piece pos ^ (r & 15), of V row r piece
+// pos ^ 4 * (r & 3).  The K operand read (16 consecutive rows, one piece) and the transposing V read (4 rows x 2 x 32
+// bytes) then each cover all 64 banks once.  Against staging through registers this removes eight LDS stores and 32
+// live registers per tile from every wave's instruction stream (-2 % run time on both benchmark shapes).
 #include "mops_common.h"
 #include <algorithm>
 #include <type_traits>
@@ -65,10 +68,11 @@ constexpr int kPD = 128;            // head dim
 constexpr int kPBM = 128;           // q rows per workgroup
 constexpr int kPBN = 64;            // kv tokens per tile
 constexpr int kPThreads = 256;
-constexpr int kPKStride = 272;      // bytes between K rows in LDS
-constexpr int kPVStride = 320;      // bytes between V rows in LDS
-constexpr int kPKTile = kPBN * kPKStride;   // 17408
-constexpr int kPVTile = kPBN * kPVStride;   // 20480
+constexpr int kPRow = 256;          // bytes of one K or V row in LDS (128 bf16, no padding)
+constexpr int kPTile = kPBN * kPRow;        // 16384: a K or V tile
+constexpr int kPKChunk = 4 * kPRow;         // a tile is 16 chunks of 4 rows
+constexpr int kPKTile = kPTile;
+constexpr int kPAhead = 4;          // LDS operand reads run this many MFMAs ahead of use
 constexpr float kLazyLog2 = 8.0f;    // the softmax reference moves when a row maximum outgrows it by this much (base-2 exponent)
 constexpr int kPCompactChunks = 4;  // the compact launch handles up to 64 * 4 sequences
 
@@ -115,9 +119,11 @@ __device__ __forceinline__ int wave_prefix_sum(int v) {
 __device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 // workgroup barrier that makes this wave's LDS traffic visible but leaves global loads in flight
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// the same once this wave's loads into LDS have landed: what the barrier publishes is the next tile
+__device__ __forceinline__ void tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPKTile + 2 * kPVTile];  // K[2] then V[2]
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kPKTile + 2 * kPTile];  // K[2] then V[2]
   __shared__ int lds_hist[kPThreads / 64][68];   // per wave: sequences by q tile count (compact launch)
   unsigned char* const lds_k = lds;
   unsigned char* const lds_v = lds + 2 * kPKTile;
@@ -273,53 +279,20 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     }
   }
 
-  // ---- cooperative tile loads: thread moves 16-byte piece (tid & 15) of rows (tid >> 4) + 16*i
-  const int ld_row = tid >> 4;
-  const int ld_slice = tid & 15;
+  // ---- cooperative tile loads, HBM -> LDS without a stop in registers (global_load_lds_dwordx4: the 64 lanes of a
+  //      wave deposit 64 x 16 bytes at consecutive LDS addresses).  Instruction i of wave w brings rows 16i + 4w .. + 3
+  //      of the tile: lane (rr = lane >> 4, pos = lane & 15) fills 16-byte position `pos` of row 16i + 4w + rr.  LDS rows
+  //      are unpadded, so bank conflicts are avoided by what a position holds: position pos of row r holds piece
+  //      pos ^ (r & 15) of a K row (the operand read of 16 consecutive rows at one piece then covers all banks) and piece
+  //      pos ^ 4 * (r & 3) of a V row (the transposing read of 4 rows x 2 x 32 bytes covers all banks).  Rows past the
+  //      end of the sequence read the sequence's last row (finite data; their scores are masked, their probabilities
+  //      zero); a tile whose cache block does not exist is filled with zeros instead.
+  const int ld_row = tid >> 4;     // 4 * wave + rr
+  const int ld_pos = tid & 15;
   const int64_t tok_elems = (int64_t)p.hkv * kPD;   // elements between tokens inside a cache block
-  const int col = g * kPD + (ld_slice << 3);
-  const uint16_t* kptr = p.k + (int64_t)(kbegin + ld_row) * p.k_ts + col;
-  const uint16_t* vptr = p.v + (int64_t)(kbegin + ld_row) * p.v_ts + col;
+  const int kcol = g * kPD + ((ld_pos ^ ld_row) << 3);
+  const int vcol = g * kPD + ((ld_pos ^ ((ld_row & 3) << 2)) << 3);
   const int32_t* table = paged ? p.block_table + (int64_t)b * p.block_table_row_stride : nullptr;
-  // returns false when the tile's cache block does not exist (table entry outside [0, num_blocks)): the tile
-  // then reads as zeros and the caller masks all of its keys
-  auto load_tile = [&](const uint16_t* base, const uint16_t* cache, int64_t ts, int tile, u32x4 (&r)[4]) -> bool {
-    const uint16_t* src;
-    bool tile_ok = true;
-    if (paged) {  // a 64-token tile lies inside one cache block (block_size is a multiple of 64)
-      const int t0 = tile * kPBN;
-      const int blk = table[t0 / p.block_size];
-      tile_ok = blk >= 0 && blk < p.num_blocks;
-      src = cache + ((int64_t)(tile_ok ? blk : 0) * p.block_size + (t0 % p.block_size) + ld_row) * tok_elems + col;
-      ts = tok_elems;
-    } else {
-      src = base + (int64_t)tile * kPBN * ts;
-    }
-    if (tile_ok && (tile + 1) * kPBN <= kv_len) {  // whole tile inside the sequence
-#pragma unroll
-      for (int i = 0; i < 4; ++i) r[i] = load16(src + (int64_t)(16 * i) * ts);
-    } else {                                        // rows past the sequence read as zeros
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int t = tile * kPBN + ld_row + 16 * i;
-        u32x4 x = {0u, 0u, 0u, 0u};
-        if (tile_ok && t < kv_len) x = load16(src + (int64_t)(16 * i) * ts);
-        r[i] = x;
-      }
-    }
-    return tile_ok;
-  };
-  const int st_k = ld_row * kPKStride + (ld_slice << 4);
-  const int st_v = ld_row * kPVStride + (ld_slice << 4);
-  auto store_k = [&](int buf, const u32x4 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds_k + buf * kPKTile + st_k + 16 * i * kPKStride) = r[i];
-  };
-  auto store_v = [&](int buf, const u32x4 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds_v + buf * kPVTile + st_v + 16 * i * kPVStride) = r[i];
-  };
-  // wave-uniform base address of a tile's first token; true when the whole tile can be loaded unconditionally
   auto tile_base = [&](const uint16_t* packed, int64_t ts, int tile, const char*& base, bool& tile_ok) -> bool {
     tile_ok = true;
     if (paged) {
@@ -332,19 +305,65 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     }
     return tile_ok && (tile + 1) * kPBN <= kv_len;
   };
-  unsigned mv_koff[4], mv_voff[4];   // this thread's byte offsets of its four pieces from a tile's base
-  {
-    const int64_t kts = paged ? tok_elems : p.k_ts, vts = paged ? tok_elems : p.v_ts;
+  // this thread's byte offset of its first piece from a tile's base; piece i lies 16 rows further
+  const unsigned k_row_bytes = (unsigned)((paged ? tok_elems : p.k_ts) * 2), v_row_bytes = (unsigned)((paged ? tok_elems : p.v_ts) * 2);
+  const unsigned mv_koff0 = (unsigned)ld_row * k_row_bytes + (unsigned)(kcol * 2);
+  const unsigned mv_voff0 = (unsigned)ld_row * v_row_bytes + (unsigned)(vcol * 2);
+  auto mv_koff = [&](int i) -> unsigned { return mv_koff0 + (unsigned)(16 * i) * k_row_bytes; };
+  auto mv_voff = [&](int i) -> unsigned { return mv_voff0 + (unsigned)(16 * i) * v_row_bytes; };
+  // Issued as inline assembly on purpose: through the compiler's builtin every later LDS read waits for the load to
+  // land (the compiler cannot tell that the buffer being filled is not the buffer being read), which would serialise
+  // the tile.  Nothing here depends on the load until the barrier at the top of the next tile, which waits for it
+  // explicitly.  M0 carries the wave's LDS destination; lane l deposits its 16 bytes at M0 + 16 * l.
+  typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
+  // M0 (the wave's LDS destination) is derived from a vector register inside the statement: a readfirstlane the
+  // compiler can see makes it treat the wave index as uniform and restructure the whole tile loop around scalar copies of
+  // everything derived from it, at the price of ~70 vector registers.  The statement opens with a wait state because
+  // on this chip a v_readfirstlane that directly follows the VALU instruction writing its source register reads the old
+  // value; the compiler spaces its own instructions accordingly but does not look inside an asm statement, and the
+  // instruction it places right before this one is usually the addition that forms the M0 value.
+  const unsigned lds_wave_base = (unsigned)(uintptr_t)(lds_ptr_t)lds + ((unsigned)(tid >> 6) << 10);
+  auto to_lds = [&](const char* base, unsigned voff, unsigned lds_off) {   // lds_off: offset of the chunk's tile and row group (wave-uniform value)
+    const char* src = base + voff;
+    unsigned m0_tmp;
+    asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %2\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 : "=&s"(m0_tmp) : "v"(src), "v"(lds_wave_base + lds_off) : "memory");
+  };
+  // offset of instruction i's 1-KiB chunk from the wave's first chunk of tile buffer 0; tile_off: offset of the tile buffer
+  auto chunk = [&](unsigned tile_off, int i) -> unsigned { return tile_off + (unsigned)(4 * i) * kPKChunk; };
+  // general form (any tile): returns false when the tile's cache block does not exist
+  auto load_tile = [&](const uint16_t* packed, int64_t ts, bool is_k, int tile, unsigned tile_off) -> bool {
+    const char* base;
+    bool tile_ok;
+    const bool whole = tile_base(packed, ts, tile, base, tile_ok);
+    const unsigned row_bytes = is_k ? k_row_bytes : v_row_bytes;
+    const unsigned colb = (unsigned)((is_k ? kcol : vcol) * 2);
+    if (!tile_ok) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mv_koff[i] = (unsigned)(((int64_t)(ld_row + 16 * i) * kts + col) * 2);
-      mv_voff[i] = (unsigned)(((int64_t)(ld_row + 16 * i) * vts + col) * 2);
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lds + tile_off + (16 * i + ld_row) * kPRow + (ld_pos << 4)) = u32x4{0u, 0u, 0u, 0u};
+    } else if (whole) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) to_lds(base, is_k ? mv_koff(i) : mv_voff(i), chunk(tile_off, i));
+    } else {
+      const int last = kv_len - 1 - tile * kPBN;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) to_lds(base, (unsigned)min(ld_row + 16 * i, last) * row_bytes + colb, chunk(tile_off, i));
     }
+    return tile_ok;
+  };
+  // K operand read: lane (n, jj) reads piece jj + 2 * k8 of row n (+ 32): at position (jj + 2 * k8) ^ (n & 15)
+  int rd_k[8];
+#pragma unroll
+  for (int k8 = 0; k8 < 8; ++k8) rd_k[k8] = n * kPRow + (((jj + 2 * k8) ^ (n & 15)) << 4);
+  // transposing V read: 16-lane group (d half, jj); lane addresses token row 4 * jj + rr2 of a 4-row set and 8 bytes of
+  // the group's 32-byte window; the 64-byte block dt of the row sits at block dt ^ rr2
+  int rd_v[4];
+  {
+    const int rr2 = (lane >> 2) & 3;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+      rd_v[dt] = (4 * jj + rr2) * kPRow + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3) + 64 * (dt ^ rr2);
   }
-  const int rd_k = n * kPKStride + (jj << 4);
-  // transposing V read: 16-lane group (d half, jj); lane addresses token row src_row of a 4-row set and
-  // the 4-wide d chunk src_chunk of the group's 16-wide window
-  const int rd_v = (4 * jj + ((lane & 15) >> 2)) * kPVStride + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3);
 
   f32x16 acc[4];
 #pragma unroll
@@ -353,7 +372,6 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
   float m_run = -INFINITY;  // running max of the raw scores of row my_row
   float l_run = 0.f;        // this lane's share of the running sum
-  u32x4 kreg[4], vreg[4];
 
   // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
   // scheduling fence are what the wave issues while that MFMA runs.
@@ -365,24 +383,25 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const int buf = tile & 1;
     f32x16 s[2];
     {
-      const unsigned char* kt = lds_k + buf * kPKTile + rd_k;
+      const unsigned char* kt = lds_k + buf * kPKTile;
+      const unsigned knext = (unsigned)(buf ^ 1) * kPKTile, vnext = 2 * kPKTile + (unsigned)(buf ^ 1) * kPTile;
       u32x4 ka[16];
-      auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + (i & 1) * 32 * kPKStride + (i >> 1) * 32); };
+      auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + rd_k[i >> 1] + (i & 1) * 32 * kPRow); };
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
-      rd(0); rd(1); rd(2); rd(3);
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
       __builtin_amdgcn_s_setprio(1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i >> 1], s[i & 1], 0, 0, 0);
-        if (i + 4 < 16) rd(i + 4);
+        if (i + kPAhead < 16) rd(i + kPAhead);
         if (decltype(move)::value && (i & 1)) {
           const int j = i >> 1;
-          if (j < 4) kreg[j] = load16(reinterpret_cast<const uint16_t*>(kbase + mv_koff[j]));
-          else vreg[j - 4] = load16(reinterpret_cast<const uint16_t*>(vbase + mv_voff[j - 4]));
+          if (j < 4) to_lds(kbase, mv_koff(j), chunk(knext, j));
+          else to_lds(vbase, mv_voff(j - 4), chunk(vnext, j - 4));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -458,33 +477,26 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int q = 0; q < 4; ++q) stage_p(q);
     // block C
     {
-      const unsigned char* vt = lds_v + buf * kPVTile + rd_v;
-      unsigned char* kdst = lds_k + (buf ^ 1) * kPKTile + st_k;
-      unsigned char* vdst = lds_v + (buf ^ 1) * kPVTile + st_v;
+      const unsigned char* vt = lds_v + buf * kPTile;
       s16x4 vlo[16], vhi[16];
       auto rd = [&](int i) {
         const int kb2 = i >> 2, dt = i & 3;
-        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + 16 * kb2 * kPVStride + 64 * dt));
-        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + (16 * kb2 + 8) * kPVStride + 64 * dt));
+        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + 16 * kb2 * kPRow));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + (16 * kb2 + 8) * kPRow));
       };
       typedef short s16x8 __attribute__((ext_vector_type(8)));
-      rd(0); rd(1); rd(2); rd(3);
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
       __builtin_amdgcn_s_setprio(1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
         acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
-        if (i + 4 < 16) rd(i + 4);
+        if (i + kPAhead < 16) rd(i + kPAhead);
         // slot i finishes pair i + 4 (needed from slot 4 * ((i + 4) / 4) on), exponentiates i + 5, scales i + 6
         if (i + 4 < 16) stage_p(i + 4);
         if (i + 5 < 16) stage_e(i + 5);
         if (i + 6 < 16) stage_f(i + 6);
-        if (decltype(move)::value && i >= 8) {
-          const int j = i - 8;
-          if (j < 4) *reinterpret_cast<u32x4*>(kdst + 16 * j * kPKStride) = kreg[j];
-          else *reinterpret_cast<u32x4*>(vdst + 16 * (j - 4) * kPVStride) = vreg[j - 4];
-        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -492,16 +504,15 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     l_run = l_run * alpha + (ps0 + ps1);
   };
 
-  // ---- tile loop.  The next tile travels HBM -> registers during block A and registers -> the other LDS
-  //      buffer during block C; that buffer was last read before this tile's barrier.
-  bool tile_exists = load_tile(kptr, p.k, p.k_ts, 0, kreg);   // the tile about to be computed has a cache block
-  load_tile(vptr, p.v, p.v_ts, 0, vreg);
+  // ---- tile loop.  The next tile travels HBM -> the other LDS buffer during block A; that buffer was last read before
+  //      this tile's barrier, and the barrier at the top of the next tile waits for the loads to have landed.
+  bool tile_exists = true;
+  if (ntiles > 0) {
+    tile_exists = load_tile(p.k, p.k_ts, true, 0, 0u);
+    load_tile(p.v, p.v_ts, false, 0, 2u * kPKTile);
+  }
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
-  if (ntiles > 0) {
-    store_k(0, kreg);
-    store_v(0, vreg);
-  }
   // Steady prefix of the loop: tiles this wave computes and whose successor is a whole tile of a packed
   // K/V.  There the per-tile bookkeeping is two pointer increments; everything else (paged caches,
   // partial tiles, the last tile, tiles this wave skips) takes the general loop below.  Both loops hold
@@ -514,7 +525,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const char* vbase = reinterpret_cast<const char*>(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
     const int64_t kstep = (int64_t)kPBN * p.k_ts * 2, vstep = (int64_t)kPBN * p.v_ts * 2;
     for (; tile < n_fast; ++tile) {
-      lds_barrier();
+      tile_barrier();
       if (tile < unmasked) tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{}, 0);
       else tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{}, my_row + shift);
       kbase += kstep;
@@ -522,39 +533,23 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     }
   }
   for (; tile < ntiles; ++tile) {
-    lds_barrier();
-    const bool have_next = tile + 1 < ntiles;
-    const char* kbase = nullptr;
-    const char* vbase = nullptr;
-    bool sliced = false, next_exists = true;
-    if (have_next && tile < my_tiles) {
-      const bool k_whole = tile_base(p.k, p.k_ts, tile + 1, kbase, next_exists);
-      const bool v_whole = tile_base(p.v, p.v_ts, tile + 1, vbase, next_exists);
-      sliced = k_whole && v_whole;
+    tile_barrier();
+    bool next_exists = true;
+    if (tile + 1 < ntiles) {
+      next_exists = load_tile(p.k, p.k_ts, true, tile + 1, (unsigned)((tile + 1) & 1) * kPKTile);
+      load_tile(p.v, p.v_ts, false, tile + 1, 2u * kPKTile + (unsigned)((tile + 1) & 1) * kPTile);
     }
     // the mask is only needed where the tile holds a key beyond the first row's horizon; a tile whose cache
-    // block does not exist (it was loaded as zeros) is masked as a whole: its keys get no weight, as in decode
+    // block does not exist (it was filled with zeros) is masked as a whole: its keys get no weight, as in decode
     const bool masked = tile * kPBN + kPBN - 1 > wave_row0 + shift || !tile_exists;
     const int horizon = tile_exists ? my_row + shift : -1;
-    if (sliced) {
-      if (masked) tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{}, horizon);
-      else tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{}, 0);
-    } else {
-      if (have_next) {
-        next_exists = load_tile(kptr, p.k, p.k_ts, tile + 1, kreg);
-        load_tile(vptr, p.v, p.v_ts, tile + 1, vreg);
-      }
-      if (tile < my_tiles) {
-        if (masked) tile_compute(tile, kbase, vbase, std::false_type{}, std::true_type{}, horizon);
-        else tile_compute(tile, kbase, vbase, std::false_type{}, std::false_type{}, 0);
-      }
-      if (have_next) {
-        store_k((tile + 1) & 1, kreg);
-        store_v((tile + 1) & 1, vreg);
-      }
+    if (tile < my_tiles) {
+      if (masked) tile_compute(tile, nullptr, nullptr, std::false_type{}, std::true_type{}, horizon);
+      else tile_compute(tile, nullptr, nullptr, std::false_type{}, std::false_type{}, 0);
     }
     tile_exists = next_exists;
   }
+  tile_barrier();   // every wave is done with the last tile: the whole of LDS is free for the epilogue
 
   // ---- epilogue.  A lane holds 8-byte pieces of its own row, which would make every store instruction
   //      touch 64 cache lines; the wave's 32 x 128 slab goes through LDS instead and leaves as whole
@@ -564,7 +559,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     constexpr int kOStride = 272;   // bytes between staged rows; 32 rows = half a K buffer
-    unsigned char* const stage = ((wave & 2) ? lds_v + (ntiles & 1) * kPVTile : lds_k + (ntiles & 1) * kPKTile) + (wave & 1) * 32 * kOStride;
+    unsigned char* const stage = lds + wave * 32 * kOStride;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
