@@ -13,7 +13,8 @@
 // MFMA opens a slot, and what the wave issues while that MFMA runs is fixed by scheduling fences
 //   block A   S^T = K . Q^T           16 x v_mfma_f32_32x32x16_bf16 per wave; Q^T stays in registers as
 //                                      the B operand; the K operand reads run four MFMAs ahead of use;
-//                                      the eight direct-to-LDS loads of the next tile ride in the slots
+//                                      the eight direct-to-LDS loads of the next tile ride in the slots,
+//                                      addressed from scalar registers (tile base, LDS destination)
 //   block B   softmax head             each lane owns one q row, so the row max is register-local
 //                                      (four v_max3 chains) plus one half-wave swap
 //                                      (v_permlane32_swap); rescale factor; the scale is folded into
@@ -329,6 +330,28 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %2\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                  : "=&s"(m0_tmp) : "v"(src), "v"(lds_wave_base + lds_off) : "memory");
   };
+  // Steady-loop form: the tile's base address and the wave's LDS destination are scalar values (no vector instruction
+  // forms an address or M0), the lane's offset from the tile base is one of eight precomputed registers.
+  auto to_lds_s = [&](uint64_t sbase, unsigned voff, unsigned lds_s) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 : : "v"(voff), "s"(sbase), "s"(lds_s) : "memory");
+  };
+  // a wave-uniform value the compiler holds in a vector register, moved to a scalar one.  Wait states on both sides,
+  // because the compiler's hazard bookkeeping does not see inside the statement: a v_readfirstlane right behind the
+  // VALU instruction that writes its source reads the old value, and a memory instruction may not take a scalar
+  // register as its base within five cycles of a VALU write to it.
+  auto to_scalar = [&](unsigned v) -> unsigned {
+    unsigned s_;
+    asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(s_) : "v"(v));
+    return s_;
+  };
+  auto to_scalar64 = [&](const void* ptr) -> uint64_t {
+    const uint64_t a = reinterpret_cast<uint64_t>(ptr);
+    return ((uint64_t)to_scalar((unsigned)(a >> 32)) << 32) | to_scalar((unsigned)a);
+  };
+  unsigned koff_r[4], voff_r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { koff_r[i] = mv_koff(i); voff_r[i] = mv_voff(i); }
   // offset of instruction i's 1-KiB chunk from the wave's first chunk of tile buffer 0; tile_off: offset of the tile buffer
   auto chunk = [&](unsigned tile_off, int i) -> unsigned { return tile_off + (unsigned)(4 * i) * kPKChunk; };
   // general form (any tile): returns false when the tile's cache block does not exist
@@ -379,12 +402,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   //   block B: row max, rescale factor, the first eight exponentials
   //   block C: O^T += V^T . P^T, the remaining exponentials and the eight LDS stores of the next tile ride in its slots
   // `horizon`: last key (sequence-relative) this lane's row may see; only read on the masked variant.
-  auto tile_compute = [&](int tile, const char* kbase, const char* vbase, auto move, auto masked, int horizon) {
+  auto tile_compute = [&](int tile, uint64_t kbase, uint64_t vbase, unsigned lds_s, auto move, auto masked, int horizon) {
     const int buf = tile & 1;
+    const unsigned lds_next = lds_s + (unsigned)((buf ^ 1) * kPKTile);
     f32x16 s[2];
     {
       const unsigned char* kt = lds_k + buf * kPKTile;
-      const unsigned knext = (unsigned)(buf ^ 1) * kPKTile, vnext = 2 * kPKTile + (unsigned)(buf ^ 1) * kPTile;
       u32x4 ka[16];
       auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + rd_k[i >> 1] + (i & 1) * 32 * kPRow); };
 #pragma unroll
@@ -400,8 +423,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         if (i + kPAhead < 16) rd(i + kPAhead);
         if (decltype(move)::value && (i & 1)) {
           const int j = i >> 1;
-          if (j < 4) to_lds(kbase, mv_koff(j), chunk(knext, j));
-          else to_lds(vbase, mv_voff(j - 4), chunk(vnext, j - 4));
+          if (j < 4) to_lds_s(kbase, koff_r[j], lds_next + (unsigned)(4 * kPKChunk * j));
+          else to_lds_s(vbase, voff_r[j - 4], lds_next + (unsigned)(2 * kPKTile + 4 * kPKChunk * (j - 4)));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -521,13 +544,14 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   if (!paged) {
     const int n_fast = min(my_tiles, min(kv_len / kPBN - 1, ntiles - 1));
     const int unmasked = wave_row0 + shift + 1 >= 0 ? (wave_row0 + shift + 1) / kPBN : 0;   // tiles wholly below the first row's horizon
-    const char* kbase = reinterpret_cast<const char*>(p.k + (int64_t)(kbegin + kPBN) * p.k_ts);
-    const char* vbase = reinterpret_cast<const char*>(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
+    uint64_t kbase = to_scalar64(p.k + (int64_t)(kbegin + kPBN) * p.k_ts);
+    uint64_t vbase = to_scalar64(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
+    const unsigned lds_s = to_scalar(lds_wave_base);
     const int64_t kstep = (int64_t)kPBN * p.k_ts * 2, vstep = (int64_t)kPBN * p.v_ts * 2;
     for (; tile < n_fast; ++tile) {
       tile_barrier();
-      if (tile < unmasked) tile_compute(tile, kbase, vbase, std::true_type{}, std::false_type{}, 0);
-      else tile_compute(tile, kbase, vbase, std::true_type{}, std::true_type{}, my_row + shift);
+      if (tile < unmasked) tile_compute(tile, kbase, vbase, lds_s, std::true_type{}, std::false_type{}, 0);
+      else tile_compute(tile, kbase, vbase, lds_s, std::true_type{}, std::true_type{}, my_row + shift);
       kbase += kstep;
       vbase += vstep;
     }
@@ -544,8 +568,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const bool masked = tile * kPBN + kPBN - 1 > wave_row0 + shift || !tile_exists;
     const int horizon = tile_exists ? my_row + shift : -1;
     if (tile < my_tiles) {
-      if (masked) tile_compute(tile, nullptr, nullptr, std::false_type{}, std::true_type{}, horizon);
-      else tile_compute(tile, nullptr, nullptr, std::false_type{}, std::false_type{}, 0);
+      if (masked) tile_compute(tile, 0, 0, 0u, std::false_type{}, std::true_type{}, horizon);
+      else tile_compute(tile, 0, 0, 0u, std::false_type{}, std::false_type{}, 0);
     }
     tile_exists = next_exists;
   }
