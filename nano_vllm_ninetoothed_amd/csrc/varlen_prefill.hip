@@ -267,19 +267,6 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   // tiles this wave has to look at: those holding a key visible to one of its rows
   const int my_tiles = max(0, min(ntiles, (wave_row0 + 31 + shift >= 0) ? (wave_row0 + 31 + shift) / kPBN + 1 : 0));
 
-  // ---- Q^T as B operand: lane (n, jj) holds Q[my_row][16*kb + 8*jj .. +8) for kb = 0..7
-  bf16x8 qb[8];
-  {
-    const bool row_ok = my_row >= 0 && my_row < seq_len;
-    const uint16_t* qrow = p.q + (int64_t)(seq_begin + (row_ok ? my_row : 0)) * p.q_ts + (int64_t)h * kPD;
-#pragma unroll
-    for (int kb = 0; kb < 8; ++kb) {
-      u32x4 w = {0u, 0u, 0u, 0u};
-      if (row_ok) w = load16(qrow + 16 * kb + 8 * jj);
-      qb[kb] = __builtin_bit_cast(bf16x8, w);
-    }
-  }
-
   // ---- cooperative tile loads, HBM -> LDS without a stop in registers (global_load_lds_dwordx4: the 64 lanes of a
   //      wave deposit 64 x 16 bytes at consecutive LDS addresses).  Instruction i of wave w brings rows 16i + 4w .. + 3
   //      of the tile: lane (rr = lane >> 4, pos = lane & 15) fills 16-byte position `pos` of row 16i + 4w + rr.  LDS rows
@@ -388,6 +375,29 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
       rd_v[dt] = (4 * jj + rr2) * kPRow + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3) + 64 * (dt ^ rr2);
   }
 
+  // ---- Q^T as B operand: lane (n, jj) holds Q[my_row][16*kb + 8*jj .. +8) for kb = 0..7.  A lane's own pieces lie 32
+  //      bytes apart, so loading them straight into registers makes every load instruction touch 32 cache lines; the
+  //      wave's 32 x 256-byte slab instead comes through LDS as eight whole-line direct loads, laid out like a K tile, into
+  //      the wave's own 8 KiB of the tile buffers that tile 0 does not use.  Only this wave reads them, and it has done so
+  //      before it reaches the first barrier, behind which the loads of tile 1 are issued.  Rows outside the sequence
+  //      take a copy of a valid row: rows are independent and theirs are never stored.
+  bf16x8 qb[8];
+  {
+    const unsigned q_lds = (unsigned)kPKTile + (unsigned)(wave & 1) * 8192u + (unsigned)(wave >> 1) * (unsigned)(2 * kPKTile);
+    const int64_t q_row_bytes = p.q_ts * 2;
+    const char* qbase = reinterpret_cast<const char*>(p.q + (int64_t)seq_begin * p.q_ts + (int64_t)h * kPD);
+    const int rr = lane >> 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int rl = 4 * i + rr;
+      const int row = min(max(wave_row0 + rl, 0), seq_len - 1);
+      const unsigned piece = (unsigned)(ld_pos ^ (rl & 15));
+      const char* src_ = qbase + (int64_t)row * q_row_bytes + piece * 16;
+      unsigned m0_tmp;
+      asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %2\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   : "=&s"(m0_tmp) : "v"(src_), "v"((unsigned)(uintptr_t)(lds_ptr_t)lds + q_lds + (unsigned)(1024 * i)) : "memory");
+    }
+  }
   f32x16 acc[4];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt)
@@ -533,6 +543,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   if (ntiles > 0) {
     tile_exists = load_tile(p.k, p.k_ts, true, 0, 0u);
     load_tile(p.v, p.v_ts, false, 0, 2u * kPKTile);
+  }
+  {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned char* qt = lds + kPKTile + (wave & 1) * 8192 + (wave >> 1) * (2 * kPKTile);
+#pragma unroll
+    for (int kb = 0; kb < 8; ++kb) qb[kb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(qt + rd_k[kb]));
   }
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
