@@ -403,7 +403,11 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
-  float m_run = -INFINITY;  // running max of the raw scores of row my_row
+  float m_run = -INFINITY;  // softmax reference of row my_row, in scaled (base-2 exponent) units
+  // the accumulator every score product starts from: minus the reference, so that the MFMA delivers score - reference
+  f32x16 s_init;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s_init[r] = 0.f;
   float l_run = 0.f;        // this lane's share of the running sum
 
   // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
@@ -420,16 +424,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
       const unsigned char* kt = lds_k + buf * kPKTile;
       u32x4 ka[16];
       auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + rd_k[i >> 1] + (i & 1) * 32 * kPRow); };
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
       for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
       __builtin_amdgcn_s_setprio(1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i >> 1], s[i & 1], 0, 0, 0);
+        s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i >> 1], i < 2 ? s_init : s[i & 1], 0, 0, 0);
         if (i + kPAhead < 16) rd(i + kPAhead);
         if (decltype(move)::value && (i & 1)) {
           const int j = i >> 1;
@@ -464,40 +464,41 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int c = 0; c < 4; ++c) mx[c] = max3(mx[c], s[c >> 1][8 * (c & 1) + 5], s[c >> 1][8 * (c & 1) + 6]);
     const float m01 = max3(mx[0], mx[1], s[0][7]), m23 = max3(mx[2], mx[3], s[0][15]);
     const float m_loc = half_swap_max(max3(m01, m23, fmaxf(s[1][7], s[1][15])));
-    // The softmax reference m_run only moves when a row's maximum outgrows it by kLazyLog2 in the exponent's base-2
-    // units: probabilities then reach at most 2^kLazyLog2 (harmless in bf16 and in the fp32 sums, and the final
-    // division by the row sum is exact for any reference), and the 64 accumulator multiplies of a rescale, behind
-    // which nothing else can be issued, run on a row's first tile or two instead of on every other tile.
+    // m_loc is relative to the reference the scores were computed against.  The reference only moves when a row's
+    // maximum outgrows it by kLazyLog2: probabilities then reach at most 2^kLazyLog2 (harmless in bf16 and in the fp32
+    // sums, and the final division by the row sum is exact for any reference), and what a move costs (64 accumulator
+    // multiplies, 32 subtractions on this tile's scores, 16 moves for s_init), behind which nothing else can be issued,
+    // runs on a row's first tile or two instead of on every other tile.
     float alpha = 1.0f;
-    const bool grow = m_loc * p.scale_log2 > m_run * p.scale_log2 + kLazyLog2;   // -inf reference: any finite maximum
+    const float m_old_safe = (m_run == -INFINITY) ? 0.f : m_run;
+    const float m_abs = m_loc + m_old_safe;
+    const bool grow = m_abs > m_run + kLazyLog2;   // -inf reference: any finite maximum
     if (__any(grow)) {
-      const float m_new = grow ? m_loc : m_run;
+      const float m_new = grow ? m_abs : m_run;
       const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_new_safe * p.scale_log2);
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new_safe);
+      const float delta = m_new_safe - m_old_safe;   // 0 in lanes whose reference stays
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[tt][r] -= delta;
       m_run = m_new;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_init[r] = -m_new_safe;
     }
-    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
-    const float mc = m_safe * p.scale_log2;
     u32x4 pw[4];   // P^T as B operand for the four 16-token k blocks
     float ps0 = 0.f, ps1 = 0.f;
     float f0[16], f1[16];   // per element pair q = 0..15 (elements 2q, 2q+1 of this lane's 32 scores): stage values
-    auto stage_f = [&](int q) {
-      const int tt = q >> 3, r = 2 * (q & 7);
-      f0[q] = __builtin_fmaf(s[tt][r], p.scale_log2, -mc);
-      f1[q] = __builtin_fmaf(s[tt][r + 1], p.scale_log2, -mc);
-    };
     auto stage_e = [&](int q) {
-      f0[q] = __builtin_amdgcn_exp2f(f0[q]);
-      f1[q] = __builtin_amdgcn_exp2f(f1[q]);
+      const int tt = q >> 3, r = 2 * (q & 7);
+      f0[q] = __builtin_amdgcn_exp2f(s[tt][r]);
+      f1[q] = __builtin_amdgcn_exp2f(s[tt][r + 1]);
     };
     auto stage_p = [&](int q) {
       const int tt = q >> 3, r = 2 * (q & 7);
       if (q & 1) ps1 += f0[q] + f1[q]; else ps0 += f0[q] + f1[q];
       pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(f0[q], f1[q]);
     };
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int q = 0; q < 6; ++q) stage_f(q);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int q = 0; q < 5; ++q) stage_e(q);
@@ -529,7 +530,6 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         // slot i finishes pair i + 4 (needed from slot 4 * ((i + 4) / 4) on), exponentiates i + 5, scales i + 6
         if (i + 4 < 16) stage_p(i + 4);
         if (i + 5 < 16) stage_e(i + 5);
-        if (i + 6 < 16) stage_f(i + 6);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -548,7 +548,15 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const unsigned char* qt = lds + kPKTile + (wave & 1) * 8192 + (wave >> 1) * (2 * kPKTile);
 #pragma unroll
-    for (int kb = 0; kb < 8; ++kb) qb[kb] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(qt + rd_k[kb]));
+    for (int kb = 0; kb < 8; ++kb) {
+      // Q is scaled by softmax_scale * log2(e) here, once, and rounded back to bf16: the scores then come out of the
+      // MFMA in the exponent's units and the softmax spends no instruction on scaling them
+      u32x4 w = *reinterpret_cast<const u32x4*>(qt + rd_k[kb]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        w[e] = pack_bf16x2(__builtin_bit_cast(float, w[e] << 16) * p.scale_log2, __builtin_bit_cast(float, w[e] & 0xffff0000u) * p.scale_log2);
+      qb[kb] = __builtin_bit_cast(bf16x8, w);
+    }
   }
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
