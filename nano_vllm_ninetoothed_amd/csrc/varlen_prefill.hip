@@ -124,8 +124,11 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kPKTile + 2 * kPTile];  // K[2] then V[2]
-  __shared__ int lds_hist[kPThreads / 64][68];   // per wave: sequences by q tile count (compact launch)
+  // One array, so that the tile buffers start at the workgroup's LDS offset 0 whatever order the compiler lays shared
+  // variables out in: a direct-to-LDS load takes its destination from M0 as a plain offset, and every tile offset here
+  // stays below 64 KiB.  K[2] then V[2], then per wave the histogram of sequences by q tile count (compact launch).
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kPKTile + 2 * kPTile + (kPThreads / 64) * 68 * 4];
+  int (*const lds_hist)[68] = reinterpret_cast<int (*)[68]>(lds + 2 * kPKTile + 2 * kPTile);
   unsigned char* const lds_k = lds;
   unsigned char* const lds_v = lds + 2 * kPKTile;
 
