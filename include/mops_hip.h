@@ -192,8 +192,9 @@ int mops_hip_attn_paged_decode_noalloc_bf16(const void* q, int64_t q_batch_strid
  *     out[i,h,:] = softmax_{j <= i + (Lk-Lq)}( scale * q[i,h,:] . K_s[j,h/(hq/hkv),:] ) @ V_s[j,h/(hq/hkv),:]
  *
  * q/out: [total_tokens, hq, 128] bf16, token strides in elements (multiples of 8), head stride 128.
- * block_table == NULL: k/v are packed [total_k_tokens, hkv, 128] with their own token strides and key j of
- *   sequence s is row cu_k[s] + j; cu_seqlens_k may be NULL (then it equals cu_seqlens_q).
+ * block_table == NULL: k/v are packed [total_k_tokens, hkv, 128] with their own token strides (multiples of 8,
+ *   at most 2^24 elements: MOPS_HIP_EUNSUPPORTED beyond) and key j of sequence s is row cu_k[s] + j;
+ *   cu_seqlens_k may be NULL (then it equals cu_seqlens_q).
  * block_table != NULL: k/v are the contiguous paged caches [num_blocks, block_size, hkv, 128] and key j of
  *   sequence s is cache[block_table[s, j/block_size], j%block_size] (row stride block_table_row_stride,
  *   at least max_blocks_per_seq columns; entries beyond the sequence's keys are never read; an entry

@@ -17,15 +17,15 @@
 //                                      addressed from scalar registers (tile base, LDS destination)
 //   block B   softmax head             each lane owns one q row, so the row max is register-local
 //                                      (four v_max3 chains) plus one half-wave swap
-//                                      (v_permlane32_swap); rescale factor; the scale is folded into
-//                                      the exponent; the causal mask is applied only on tiles that
-//                                      reach past the wave's first row
+//                                      (v_permlane32_swap); Q carries softmax_scale * log2(e) and the
+//                                      score MFMAs start from minus the row's reference, so the scores
+//                                      arrive as exponents; the reference moves lazily; the causal mask
+//                                      is applied only on tiles that reach past the wave's first row
 //   block C   O^T += V^T . P^T         16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
 //                                      already the B-operand layout, V^T comes out of LDS through
 //                                      ds_read_b64_tr_b16 four MFMAs ahead; the exponent pipeline
-//                                      (scale, exp2, sum and pack), skewed one slot per stage, rides in
-//                                      the slots
-// In the steady part of the tile loop the per-tile bookkeeping is two pointer increments.
+//                                      (exp2, sum and pack), skewed one slot per stage, rides in the slots
+// In the steady part of the tile loop the per-tile bookkeeping is two scalar additions.
 //
 // What was measured on this part and shaped the kernel:
 //   * A wave issues a VALU instruction every ~5 cycles (a dependent one every ~9, an exp2 every ~8);
@@ -35,8 +35,9 @@
 //   * Address and bounds bookkeeping between the barrier and the first MFMA took ~900 cycles per tile
 //     (a quarter of the tile) before the steady loop replaced it by pointer increments.
 //   * Issued in one burst after the barrier, the eight 1-KiB global loads of a wave took ~200 cycles
-//     each to issue (all eight waves of the CU queue on the same address path) and the eight LDS stores
-//     ~60 cycles each; spread over the MFMA slots both costs vanish behind the matrix pipe.
+//     each to issue (all eight waves of the CU queue on the same address path); spread over the MFMA
+//     slots the cost vanishes behind the matrix pipe.  Forming a load's address and M0 with vector
+//     instructions cost 8 % of the run time; both come from scalar registers now.
 //   * Every VALU read of an MFMA result goes through compiler-visible code: the wait states between an
 //     MFMA and the first read of its result are software-inserted, and an inline-assembly v_max3 on the
 //     scores read half-written registers now and then (results then differ by an ulp from run to run).
@@ -45,13 +46,18 @@
 //     8192-token sequences, -10 % on 128..2048-token ones), one wave per SIMD owning two 32-row slabs
 //     (512 registers; the compiler shuttles values between the two register files), software-pipelining
 //     the two products across half tiles inside a wave (register pressure, two barriers per tile).
-//   * Per workgroup there is a fixed cost of ~7 us next to ~2 us per tile: rank -> tile mapping, Q and
-//     first-tile loads, the epilogue, and the gap until the dispatcher starts the successor.  A persistent
-//     launch (resident workgroups drawing items by ticket) did not shrink it (it is dependent latency, not
-//     dispatch time) and lengthened the tail; it was 6 % slower on 128..2048-token sequences.
-//   * The transposing read ds_read_b64_tr_b16 delivers ~65 B/clk per CU against ~210 B/clk for
-//     ds_read_b128, but replacing it by plain reads of a pre-transposed tile changed the run time by
-//     2 %: the LDS pipe is not what bounds this shape.
+//   * Per workgroup there is a fixed cost of ~6.7 us next to ~1.7 - 2.1 us per tile: rank -> tile mapping
+//     (1.1 us), issuing the Q and first-tile loads (1.6 us: ~240 cycles per load instruction while the
+//     CU's other workgroup streams its tiles), their landing (1 us), the epilogue (1.1 us).  It is the
+//     issue of vector-memory instructions, not the latency of the data: pulling the successor's Q into
+//     L2 ahead of time made it longer.  A persistent launch (resident workgroups drawing items by
+//     ticket) did not shrink it and lengthened the tail; it was 6 % slower on 128..2048-token sequences.
+//   * With four waves per CU the transposing read ds_read_b64_tr_b16 delivers ~97 B/clk per CU, a plain
+//     ds_read_b64 ~120, ds_read_b128 ~167; each wave reads the whole 16 KiB V tile, and block C's
+//     ~1000 cycles track those reads.  With 32 query rows per wave an MFMA consumes 1 KiB of LDS operand
+//     per 32 cycles: LDS read bandwidth and matrix rate saturate together.
+//   * The shader clock falls to ~1.5 GHz under this kernel on 8192-token sequences (s_memtime against
+//     the 100 MHz wall clock; 2.4 GHz idle): counted in cycles the matrix pipe is 72 % busy there.
 //
 // K/V tiles travel HBM -> LDS directly (global_load_lds_dwordx4, no stop in registers), so LDS rows are unpadded
 // (256 B, the two double-buffered tile pairs fill exactly 64 KiB) and bank conflicts are avoided by a swizzle applied
@@ -665,6 +671,8 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   } else {
     if (k_token_stride < hkv * kPD || v_token_stride < hkv * kPD) return MOPS_HIP_EINVAL;
     if ((k_token_stride & 7) || (v_token_stride & 7)) return MOPS_HIP_EALIGN;
+    // a lane's byte offset inside a 64-token tile is kept in 32 bits
+    if (k_token_stride > (1ll << 24) || v_token_stride > (1ll << 24)) return MOPS_HIP_EUNSUPPORTED;
     if (!cu_seqlens_k && total_k_tokens != total_tokens) return MOPS_HIP_EINVAL;
   }
   if (max_seqlen_q > total_tokens) max_seqlen_q = total_tokens;
