@@ -41,7 +41,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "prefill_long", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
+                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
@@ -275,6 +275,35 @@ def main():
                 ts.append(time.perf_counter() - t0)
             return sorted(ts)[1], "whole batch, median of 3", work
 
+    elif args.op == "prefix_prefill":
+        # prefix-cache hit (nanovllm/layers/attention.py:32-33 of the reference): 16 sequences with 1024 tokens already in
+        # the paged cache and 1024 new ones; keys are read through block_table
+        new, prefix = [1024] * 16, [1024] * 16
+        d = W.to_device(W.prefix_prefill_inputs(new, prefix, seed=args.seed, poison_unused=False), dev)
+        op = mops.flash_attn_varlen_func
+
+        def step(i):
+            return op(d["q"], d["k_cache"], d["v_cache"], max_seqlen_q=d["max_seqlen_q"], cu_seqlens_q=d["cu_seqlens_q"],
+                      max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"], softmax_scale=d["scale"], causal=True,
+                      block_table=d["block_table"])
+
+        work = float(sum(4 * 128 * 16 * (n * pl + n * (n + 1) // 2) for n, pl in zip(new, prefix)))
+        bound = "mfma"
+        metric, unit = "varlen_prefill_attn_TFLOPs", "TFLOP/s"
+        config = {"workload": "varlen causal prefill behind a cached prefix, keys in the paged cache, Qwen3-0.6B shape", "batch": 16,
+                  "q_heads": 16, "kv_heads": 8, "head_dim": 128, "new_tokens": "16 x 1024", "cached_prefix": "16 x 1024",
+                  "block_size": W.BLOCK_SIZE}
+        kernel_name = "varlen_prefill_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("flash_attn_varlen_func", "torch")
+            c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+            t0 = time.perf_counter()
+            ref(c["q"][:1024], c["k_cache"], c["v_cache"], max_seqlen_q=1024, cu_seqlens_q=c["cu_seqlens_q"][:2], max_seqlen_k=2048,
+                cu_seqlens_k=c["cu_seqlens_k"][:2], softmax_scale=c["scale"], causal=True, block_table=c["block_table"][:1])
+            return time.perf_counter() - t0, "first of the 16 sequences, one run", work / 16
+
     elif args.op == "store":
         lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
         T = sum(lens)
@@ -433,7 +462,7 @@ def main():
         cval = units / secs / (1e9 if bound == "hbm" else 1e12)
         out["cpu_baseline"] = {"value": round(cval, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
                                "sample": sample, "seconds": round(secs, 4)}
-    if args.op in ("prefill", "prefill_long"):
+    if args.op in ("prefill", "prefill_long", "prefix_prefill"):
         # what a library bf16 GEMM sustains on this chip in this run: the 2.5 PFLOP/s peak assumes 2.4 GHz, which the
         # part does not hold under matrix load, so this is the practical MFMA ceiling to read the fraction against
         n = 8192

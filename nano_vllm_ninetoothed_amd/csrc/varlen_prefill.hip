@@ -569,24 +569,56 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   }
 #pragma unroll
   for (int kb = 0; kb < 8; ++kb) asm volatile("" : "+v"(qb[kb]));
-  // Steady prefix of the loop: tiles this wave computes and whose successor is a whole tile of a packed
-  // K/V.  There the per-tile bookkeeping is two pointer increments; everything else (paged caches,
-  // partial tiles, the last tile, tiles this wave skips) takes the general loop below.  Both loops hold
+  // Steady prefix of the loop: tiles this wave computes and whose successor is a whole tile.  There the
+  // per-tile bookkeeping is two scalar additions; everything else (partial tiles, the last tile, tiles this
+  // wave skips, paged sequences of more than 64 blocks or with a missing block) takes the general loop below.  Both loops hold
   // exactly one barrier per tile, so the waves of a workgroup may sit in different ones.
   int tile = 0;
-  if (!paged) {
-    const int n_fast = min(my_tiles, min(kv_len / kPBN - 1, ntiles - 1));
+  {
+    // Paged caches take the steady loop when the sequence's keys lie in at most 64 cache blocks, all of which exist:
+    // lane l holds block l's table entry, a tile's base comes out of it by a lane read (a scalar value, no trip to
+    // memory inside the loop), and inside a block the base advances by one tile's bytes.
+    int entry = 0;
+    bool steady = true;
+    int tiles_per_block = 1;
+    if (paged) {
+      const int used_blocks = (kv_len + p.block_size - 1) / p.block_size;
+      if (lane < used_blocks) entry = table[lane];   // used_blocks > 64: not taken below
+      const bool entry_ok = lane >= used_blocks || (entry >= 0 && entry < p.num_blocks);
+      steady = used_blocks <= 64 && __all(entry_ok);
+      tiles_per_block = p.block_size / kPBN;
+    }
+    const int n_fast = steady ? min(my_tiles, min(kv_len / kPBN - 1, ntiles - 1)) : 0;
     const int unmasked = wave_row0 + shift + 1 >= 0 ? (wave_row0 + shift + 1) / kPBN : 0;   // tiles wholly below the first row's horizon
-    uint64_t kbase = to_scalar64(p.k + (int64_t)(kbegin + kPBN) * p.k_ts);
-    uint64_t vbase = to_scalar64(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
+    // byte distance between consecutive tiles of a packed K / V, or of a cache block
+    const uint64_t kstep = (uint64_t)kPBN * (uint64_t)(paged ? tok_elems : p.k_ts) * 2u, vstep = (uint64_t)kPBN * (uint64_t)(paged ? tok_elems : p.v_ts) * 2u;
+    const uint64_t block_bytes = (uint64_t)p.block_size * (uint64_t)tok_elems * 2u;
     const unsigned lds_s = to_scalar(lds_wave_base);
-    const int64_t kstep = (int64_t)kPBN * p.k_ts * 2, vstep = (int64_t)kPBN * p.v_ts * 2;
+    // base of the tile after the one being computed (tile 1 to begin with)
+    uint64_t kbase, vbase;
+    int blk_i = 1 / tiles_per_block, in_blk = 1 % tiles_per_block;
+    if (paged) {
+      const uint64_t off = (uint64_t)(unsigned)__builtin_amdgcn_readlane(entry, blk_i & 63) * block_bytes + (uint64_t)in_blk * kstep;
+      kbase = reinterpret_cast<uint64_t>(p.k) + off;
+      vbase = reinterpret_cast<uint64_t>(p.v) + off;
+    } else {
+      kbase = to_scalar64(p.k + (int64_t)(kbegin + kPBN) * p.k_ts);
+      vbase = to_scalar64(p.v + (int64_t)(kbegin + kPBN) * p.v_ts);
+    }
     for (; tile < n_fast; ++tile) {
       tile_barrier();
       if (tile < unmasked) tile_compute(tile, kbase, vbase, lds_s, std::true_type{}, std::false_type{}, 0);
       else tile_compute(tile, kbase, vbase, lds_s, std::true_type{}, std::true_type{}, my_row + shift);
-      kbase += kstep;
-      vbase += vstep;
+      if (paged && ++in_blk == tiles_per_block) {
+        in_blk = 0;
+        ++blk_i;
+        const uint64_t off = (uint64_t)(unsigned)__builtin_amdgcn_readlane(entry, blk_i & 63) * block_bytes;
+        kbase = reinterpret_cast<uint64_t>(p.k) + off;
+        vbase = reinterpret_cast<uint64_t>(p.v) + off;
+      } else {
+        kbase += kstep;
+        vbase += vstep;
+      }
     }
   }
   for (; tile < ntiles; ++tile) {
@@ -627,7 +659,10 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         *reinterpret_cast<u32x2*>(stage + n * kOStride + 64 * dt + 16 * rq + 8 * jj) = w;
       }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes, read back by other lanes
-    const int piece = lane & 15, row4 = lane >> 4;
+    int piece = lane & 15, row4 = lane >> 4;
+    // opaque to the compiler on purpose: otherwise it recognises the row numbers of the Q loads at the top of the kernel
+    // and keeps eight registers of them alive through the tile loop
+    asm volatile("" : "+v"(piece), "+v"(row4));
     uint16_t* const obase = p.out + (int64_t)(seq_begin + wave_row0) * p.o_ts + (int64_t)h * kPD + 8 * piece;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {

@@ -139,6 +139,26 @@ def test_prefill_with_cached_prefix_matches_oracle(gpu, ops, new, prefix, hq, hk
     assert_bit_exact(got_packed, got, "packed keys with cu_seqlens_k vs paged keys")
 
 
+@pytest.mark.parametrize("block_size,new,prefix", [
+    (64, [300, 70], [200, 1000]), (128, [129, 640], [127, 900]), (512, [700], [1500]),
+    (64, [200], [4300]),     # 71 cache blocks: more than the 64 table entries a wave keeps in registers
+    (256, [500, 300], [16500, 100])])
+def test_prefill_with_cached_prefix_other_block_sizes_and_long_tables(gpu, ops, monkeypatch, block_size, new, prefix):
+    """The steady part of the tile loop steps through a cache block tile by tile and takes the next block's table entry
+    from a register (up to 64 blocks per sequence); other block sizes change how many tiles a block holds, and
+    sequences with more blocks take the general loop for every tile."""
+    hip, ref = ops("flash_attn_varlen_func")
+    monkeypatch.setattr(W, "BLOCK_SIZE", block_size)
+    d = W.prefix_prefill_inputs(new, prefix, hq=4, hkv=2, seed=block_size + sum(new))
+    assert d["k_cache"].shape[1] == block_size
+    want = ref(d["q"], torch.nan_to_num(d["k_cache"]), torch.nan_to_num(d["v_cache"]), max_seqlen_q=d["max_seqlen_q"],
+               cu_seqlens_q=d["cu_seqlens_q"], max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"],
+               softmax_scale=d["scale"], causal=True, block_table=d["block_table"])
+    got = _run_prefix(hip, d, gpu, paged=True)
+    assert_attention_close(got, want, f"paged prefix prefill, block size {block_size}, new={new} prefix={prefix}")
+    assert_bit_exact(_run_prefix(hip, d, gpu, paged=False), got, "packed keys with cu_seqlens_k vs paged keys")
+
+
 def test_prefix_prefill_treats_a_missing_block_as_empty(gpu, ops):
     """A block_table entry outside [0, num_blocks) inside the used range: the keys of that block get no weight (the
     rule paged decode follows for the same metadata), instead of entering the softmax with score 0."""
