@@ -546,6 +546,110 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     l_run = l_run * alpha + (ps0 + ps1);
   };
 
+  // The same for a tile of which no row of this wave sees more than the first 32 keys (a wave's last tile on the
+  // diagonal, every other time): the fully masked half is neither multiplied nor exponentiated.  Eight MFMAs per block.
+  auto tile_compute_half = [&](int tile, uint64_t kbase, uint64_t vbase, unsigned lds_s, auto move, int horizon) {
+    const int buf = tile & 1;
+    const unsigned lds_next = lds_s + (unsigned)((buf ^ 1) * kPKTile);
+    f32x16 s0;
+    {
+      const unsigned char* kt = lds_k + buf * kPKTile;
+      u32x4 ka[8];
+      auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + rd_k[i]); };
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i], i == 0 ? s_init : s0, 0, 0, 0);
+        if (i + kPAhead < 8) rd(i + kPAhead);
+        if (decltype(move)::value) {
+          if (i < 4) to_lds_s(kbase, koff_r[i], lds_next + (unsigned)(4 * kPKChunk * i));
+          else to_lds_s(vbase, voff_r[i - 4], lds_next + (unsigned)(2 * kPKTile + 4 * kPKChunk * (i - 4)));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    {
+      const int j0 = tile * kPBN;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = j0 + 8 * (r >> 2) + 4 * jj + (r & 3);
+        s0[r] = key <= horizon ? s0[r] : -INFINITY;
+      }
+    }
+    float mx[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mx[c] = max3(s0[8 * c], s0[8 * c + 1], s0[8 * c + 2]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mx[c] = max3(mx[c], s0[8 * c + 3], s0[8 * c + 4]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mx[c] = max3(mx[c], s0[8 * c + 5], s0[8 * c + 6]);
+    const float m_loc = half_swap_max(max3(mx[0], mx[1], fmaxf(s0[7], s0[15])));
+    float alpha = 1.0f;
+    const float m_old_safe = (m_run == -INFINITY) ? 0.f : m_run;
+    const float m_abs = m_loc + m_old_safe;
+    const bool grow = m_abs > m_run + kLazyLog2;
+    if (__any(grow)) {
+      const float m_new = grow ? m_abs : m_run;
+      const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new_safe);
+      const float delta = m_new_safe - m_old_safe;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s0[r] -= delta;
+      m_run = m_new;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_init[r] = -m_new_safe;
+    }
+    u32x4 pw[2];
+    float ps0 = 0.f, ps1 = 0.f;
+    float f0[8], f1[8];
+    auto stage_e = [&](int q) {
+      f0[q] = __builtin_amdgcn_exp2f(s0[2 * q]);
+      f1[q] = __builtin_amdgcn_exp2f(s0[2 * q + 1]);
+    };
+    auto stage_p = [&](int q) {
+      const int r = 2 * q;
+      if (q & 1) ps1 += f0[q] + f1[q]; else ps0 += f0[q] + f1[q];
+      pw[r >> 3][(r & 7) >> 1] = pack_bf16x2(f0[q], f1[q]);
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < 5; ++q) stage_e(q);
+    __builtin_amdgcn_sched_barrier(0);
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_p(q);
+    {
+      const unsigned char* vt = lds_v + buf * kPTile;
+      s16x4 vlo[8], vhi[8];
+      auto rd = [&](int i) {
+        const int kb2 = i >> 2, dt = i & 3;
+        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + 16 * kb2 * kPRow));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + (16 * kb2 + 8) * kPRow));
+      };
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
+        if (i + kPAhead < 8) rd(i + kPAhead);
+        if (i + 4 < 8) stage_p(i + 4);
+        if (i + 5 < 8) stage_e(i + 5);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    l_run = l_run * alpha + (ps0 + ps1);
+  };
+
   // ---- tile loop.  The next tile travels HBM -> the other LDS buffer during block A; that buffer was last read before
   //      this tile's barrier, and the barrier at the top of the next tile waits for the loads to have landed.
   bool tile_exists = true;
@@ -608,6 +712,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (; tile < n_fast; ++tile) {
       tile_barrier();
       if (tile < unmasked) tile_compute(tile, kbase, vbase, lds_s, std::true_type{}, std::false_type{}, 0);
+      else if (wave_row0 + 31 + shift < tile * kPBN + 32) tile_compute_half(tile, kbase, vbase, lds_s, std::true_type{}, my_row + shift);
       else tile_compute(tile, kbase, vbase, lds_s, std::true_type{}, std::true_type{}, my_row + shift);
       if (paged && ++in_blk == tiles_per_block) {
         in_blk = 0;
@@ -633,7 +738,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const bool masked = tile * kPBN + kPBN - 1 > wave_row0 + shift || !tile_exists;
     const int horizon = tile_exists ? my_row + shift : -1;
     if (tile < my_tiles) {
-      if (masked) tile_compute(tile, 0, 0, 0u, std::false_type{}, std::true_type{}, horizon);
+      if (tile_exists && wave_row0 + 31 + shift < tile * kPBN + 32) tile_compute_half(tile, 0, 0, 0u, std::false_type{}, horizon);
+      else if (masked) tile_compute(tile, 0, 0, 0u, std::false_type{}, std::true_type{}, horizon);
       else tile_compute(tile, 0, 0, 0u, std::false_type{}, std::false_type{}, 0);
     }
     tile_exists = next_exists;
