@@ -774,7 +774,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     for (int i = 0; i < 8; ++i) {
       const int row = row4 + 4 * i;
       const u32x4 w = *reinterpret_cast<const u32x4*>(stage + row * kOStride + 16 * piece);
-      if (wave_row0 + row >= 0 && wave_row0 + row < seq_len) *reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts) = w;
+      // written once and not read again here: a streaming store leaves less for the write-back at the end of the kernel
+      if (wave_row0 + row >= 0 && wave_row0 + row < seq_len) __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts));
     }
   }
 }
