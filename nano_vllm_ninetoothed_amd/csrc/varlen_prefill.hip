@@ -245,8 +245,13 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     m = p.m_tiles - 1 - rest / p.batch;
     seq_begin = p.cu_seqlens[b];
     seq_end = p.cu_seqlens[b + 1];
-    kbegin = p.cu_seqlens_k[b];
-    kend = p.cu_seqlens_k[b + 1];
+    if (p.cu_seqlens_k == p.cu_seqlens) {
+      kbegin = seq_begin;
+      kend = seq_end;
+    } else {
+      kbegin = p.cu_seqlens_k[b];
+      kend = p.cu_seqlens_k[b + 1];
+    }
   }
   const int seq_len = min(seq_end, p.total_tokens) - seq_begin;   // query rows of this sequence
   // q tiles are aligned to the END of the sequence: tile m covers rows [q0, q0 + 128) with q0 = len - 128 * (tiles - m),
