@@ -124,9 +124,7 @@ __device__ __forceinline__ int wave_prefix_sum(int v) {
 // operation: the wait states between an MFMA and the first VALU read of its result are inserted by the
 // compiler's hazard recognizer, which does not look inside inline assembly.
 __device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
-// workgroup barrier that makes this wave's LDS traffic visible but leaves global loads in flight
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-// the same once this wave's loads into LDS have landed: what the barrier publishes is the next tile
+// workgroup barrier once this wave's LDS traffic is done and its loads into LDS have landed: what it publishes is the next tile
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
@@ -426,9 +424,9 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 
   // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
   // scheduling fence are what the wave issues while that MFMA runs.
-  //   block A: S^T = K . Q^T, the eight global loads of the next tile ride in its slots
-  //   block B: row max, rescale factor, the first eight exponentials
-  //   block C: O^T += V^T . P^T, the remaining exponentials and the eight LDS stores of the next tile ride in its slots
+  //   block A: S^T = K . Q^T, the eight direct-to-LDS loads of the next tile ride in its slots
+  //   block B: row max, whether the reference has to move, the first ten exponentials
+  //   block C: O^T += V^T . P^T, the remaining exponentials, the row sums and the bf16 packing ride in its slots
   // `horizon`: last key (sequence-relative) this lane's row may see; only read on the masked variant.
   auto tile_compute = [&](int tile, uint64_t kbase, uint64_t vbase, unsigned lds_s, auto move, auto masked, int horizon) {
     const int buf = tile & 1;
@@ -467,8 +465,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     }
     // A wave issues in order and a dependent VALU instruction waits ~20 cycles for its operand, so the
     // softmax is written for instruction-level parallelism: four max chains, and the exponent pipeline
-    // F (scale and subtract) -> E (exp2) -> P (row sum, bf16 pack) is skewed by one MFMA slot per stage,
-    // so nothing issued in a slot depends on anything else issued in it.
+    // E (exp2) -> P (row sum, bf16 pack) is skewed by one MFMA slot per stage, so nothing issued in a slot
+    // depends on anything else issued in it.
     float mx[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) mx[c] = max3(s[c >> 1][8 * (c & 1)], s[c >> 1][8 * (c & 1) + 1], s[c >> 1][8 * (c & 1) + 2]);
@@ -541,7 +539,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
         const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
         acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
         if (i + kPAhead < 16) rd(i + kPAhead);
-        // slot i finishes pair i + 4 (needed from slot 4 * ((i + 4) / 4) on), exponentiates i + 5, scales i + 6
+        // slot i finishes pair i + 4 (needed from slot 4 * ((i + 4) / 4) on) and exponentiates pair i + 5
         if (i + 4 < 16) stage_p(i + 4);
         if (i + 5 < 16) stage_e(i + 5);
         __builtin_amdgcn_sched_barrier(0);
@@ -753,12 +751,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
 
   // ---- epilogue.  A lane holds 8-byte pieces of its own row, which would make every store instruction
   //      touch 64 cache lines; the wave's 32 x 128 slab goes through LDS instead and leaves as whole
-  //      256-byte rows, four per store instruction.  The staging area is the K/V buffer pair the last
-  //      tile did not use: no wave reads it any more once all have passed the last tile's barrier.
+  //      256-byte rows, four per store instruction.  The staging area is the start of the tile buffers:
+  //      no wave reads a tile any more once all have passed the barrier above.
   l_run = half_swap_sum(l_run);
   {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    constexpr int kOStride = 272;   // bytes between staged rows; 32 rows = half a K buffer
+    constexpr int kOStride = 272;   // bytes between staged rows (padded: the 8-byte pieces of 32 rows spread over the banks)
     unsigned char* const stage = lds + wave * 32 * kOStride;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
