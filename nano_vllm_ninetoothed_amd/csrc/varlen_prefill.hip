@@ -331,6 +331,9 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   };
   // Steady-loop form: the tile's base address and the wave's LDS destination are scalar values (no vector instruction
   // forms an address or M0), the lane's offset from the tile base is one of eight precomputed registers.
+  // Both scalar operands are products of scalar arithmetic at every call site (to_scalar() below pays the wait states a
+  // VALU-written scalar register needs before a memory instruction may read it); five wait states here instead of one
+  // would make the statement safe for any operand and cost 1 % of the run time.
   auto to_lds_s = [&](uint64_t sbase, unsigned voff, unsigned lds_s) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  : : "v"(voff), "s"(sbase), "s"(lds_s) : "memory");
