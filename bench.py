@@ -41,7 +41,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "add_rms", "rms", "embedding", "copy", "e2e"])
+                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "silu", "sampler", "qk_rope_store", "add_rms", "rms", "embedding", "copy", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
@@ -372,6 +372,96 @@ def main():
                 ref(*a)
                 ts.append(time.perf_counter() - t0)
             return sorted(ts)[3], "whole batch, median of 7", work
+
+    elif args.op == "silu":
+        # siluAndMul on the gate_up buffer of a 16384-token prefill step (intermediate 3072); x and y are its two halves
+        rows, inter, n_copies = 16384, 3072, 4
+        bufs = [torch.randn((rows, 2 * inter), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(n_copies)]
+        op = mops.get_op("siluAndMul", "hip")
+
+        def step(i):
+            x, y = bufs[i % n_copies].chunk(2, dim=-1)
+            return op(x, y)
+
+        work = float(rows * 3 * inter * 2)
+        metric, unit = "silu_and_mul_GBps", "GB/s"
+        config = {"workload": "siluAndMul, 16384 tokens x intermediate 3072 (Qwen3-0.6B), halves of one gate_up buffer", "rows": rows,
+                  "intermediate": inter, "buffers_rotated": n_copies}
+        kernel_name = "silu_and_mul_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("siluAndMul", "torch")
+            x, y = bufs[0].cpu().chunk(2, dim=-1)
+            ts = []
+            for _ in range(5):
+                t0 = time.perf_counter()
+                ref(x, y)
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[2], "whole batch, median of 5", work
+
+    elif args.op == "sampler":
+        # sampler_forward on the logits of a 256-sequence decode step (vocab 151936)
+        rows, vocab, n_copies = 256, 151936, 4
+        logit_sets = [torch.randn((rows, vocab), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(n_copies)]
+        temps = torch.full((rows,), 0.6, device=dev)
+        op = mops.get_op("sampler_forward", "hip")
+
+        def step(i):
+            return op(logit_sets[i % n_copies], temps)
+
+        work = float(rows * vocab * 2 + rows * 8)
+        metric, unit = "sampler_GBps", "GB/s"
+        config = {"workload": "sampler_forward (greedy: row argmax), 256 rows x vocab 151936 bf16 logits", "rows": rows, "vocab": vocab,
+                  "buffers_rotated": n_copies}
+        kernel_name = "row_argmax_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("sampler_forward", "torch")
+            lg, tp = logit_sets[0].cpu(), temps.cpu()
+            ts = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                ref(lg, tp)
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[1], "whole batch, median of 3", work
+
+    elif args.op == "qk_rope_store":
+        # the fused q_norm + k_norm + rotary + store_kvcache launch on the qkv buffer of the cfg2 token count
+        lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
+        T, hq, hkv, hd, n_copies = sum(lens), 16, 8, 128, 4
+        nblk = (T + 255) // 256 + 2
+        sets = []
+        for i in range(n_copies):
+            qkv = torch.randn((T, (hq + 2 * hkv) * hd), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            sets.append({"qkv": qkv, "kc": torch.zeros((nblk, 256, hkv, hd), dtype=torch.bfloat16, device=dev),
+                         "vc": torch.zeros((nblk, 256, hkv, hd), dtype=torch.bfloat16, device=dev),
+                         "slots": torch.randperm(nblk * 256, generator=g, device=dev)[:T].to(torch.int32)})
+        qw = (1 + 0.1 * torch.randn(hd, generator=g, device=dev)).to(torch.bfloat16)
+        kw = (1 + 0.1 * torch.randn(hd, generator=g, device=dev)).to(torch.bfloat16)
+        ang = torch.rand((T, 1, hd // 2), generator=g, device=dev) * 6.28
+        cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
+        op = mops.get_op("qk_norm_rope_store", "hip")
+
+        def step(i):
+            st = sets[i % n_copies]
+            return op(st["qkv"], qw, kw, 1e-6, cos, sin, st["kc"], st["vc"], st["slots"], hq, hkv, need_k=False)
+
+        # read q, k, v rows, cos, sin and the slot; write q, the rotated k and v into the caches
+        work = float(T * ((hq + 2 * hkv) * hd * 2 + 2 * (hd // 2) * 4 + 4 + hq * hd * 2 + 2 * hkv * hd * 2))
+        metric, unit = "qk_norm_rope_store_GBps", "GB/s"
+        config = {"workload": "fused q_norm + k_norm + rotary + store_kvcache, cfg2 token count, Qwen3-0.6B heads", "tokens": T,
+                  "q_heads": hq, "kv_heads": hkv, "head_dim": hd, "buffers_rotated": n_copies}
+        kernel_name = "qk_norm_rope_store_kernel"
+
+        def cpu_fn():
+            import oracle.mops_torch  # noqa: F401
+            ref = mops.get_op("qk_norm_rope_store", "torch")
+            st = {k: v.cpu() for k, v in sets[0].items()}
+            t0 = time.perf_counter()
+            ref(st["qkv"], qw.cpu(), kw.cpu(), 1e-6, cos.cpu(), sin.cpu(), st["kc"], st["vc"], st["slots"], hq, hkv, need_k=False)
+            return time.perf_counter() - t0, "whole batch, one run", work
 
     elif args.op == "copy":
         nbytes = 1 << 30

@@ -148,8 +148,7 @@ __global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16
   // A NaN or +inf logit turns the whole softmax row into NaN, and the library's argmax of an all-NaN row is 0.
   bool spoiled = false;
   const int pieces = n >> 3;
-  for (int pc = threadIdx.x; pc < pieces; pc += kArgmaxThreads) {
-    const u32x4 w = load16_stream(row + (pc << 3));
+  auto take = [&](const u32x4 w, int pc) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float lo = bf16lo_to_f32(w[e]), hi = bf16hi_to_f32(w[e]);
@@ -158,7 +157,18 @@ __global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16
       if (lo > bv) { bv = lo; bi = i0; }        // strictly greater: within a lane indices only grow
       if (hi > bv) { bv = hi; bi = i0 + 1; }
     }
+  };
+  // four loads in flight per lane (eight are slower again): one workgroup per row leaves the memory system too little to do otherwise
+  constexpr int kDeep = 4;
+  int pc = threadIdx.x;
+  for (; pc + (kDeep - 1) * kArgmaxThreads < pieces; pc += kDeep * kArgmaxThreads) {
+    u32x4 w[kDeep];
+#pragma unroll
+    for (int u = 0; u < kDeep; ++u) w[u] = load16_stream(row + ((int64_t)(pc + u * kArgmaxThreads) << 3));
+#pragma unroll
+    for (int u = 0; u < kDeep; ++u) take(w[u], pc + u * kArgmaxThreads);
   }
+  for (; pc < pieces; pc += kArgmaxThreads) take(load16_stream(row + ((int64_t)pc << 3)), pc);
   for (int i = (pieces << 3) + threadIdx.x; i < n; i += kArgmaxThreads) {  // tail when n % 8 != 0
     const float x = bf16lo_to_f32(row[i]);
     spoiled |= !(x < INFINITY);
