@@ -201,7 +201,10 @@ int mops_hip_attn_paged_decode_noalloc_bf16(const void* q, int64_t q_batch_strid
  *   outside [0, num_blocks) inside the used range is treated as an empty block, i.e. its keys get no weight,
  *   the rule of the decode entry points; block_size must be a multiple of 64); k/v token strides are ignored.
  * cu_seqlens_*: int32 [batch+1], non-decreasing, starting at 0.  max_seqlen_q bounds every query length
- * and only sizes the launch.  Sequences of length 0 are allowed.
+ * and only sizes the launch.  Sequences of length 0 are allowed.  softmax_scale may be any finite value
+ * (0: uniform weights over the visible keys).  The scale is applied to the fp32 scores in fp32; with
+ * MOPS_HIP_PREFILL_PRESCALE=1 in the environment (read at the first call) Q is multiplied by
+ * softmax_scale * log2(e) once and rounded back to bf16 instead: faster, less accurate for large scores.
  */
 int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_stride,
                                      const void* k, int64_t k_token_stride,

@@ -17,14 +17,14 @@
 //                                      addressed from scalar registers (tile base, LDS destination)
 //   block B   softmax head             each lane owns one q row, so the row max is register-local
 //                                      (four v_max3 chains) plus one half-wave swap
-//                                      (v_permlane32_swap); Q carries softmax_scale * log2(e) and the
-//                                      score MFMAs start from minus the row's reference, so the scores
-//                                      arrive as exponents; the reference moves lazily; the causal mask
-//                                      is applied only on tiles that reach past the wave's first row
+//                                      (v_permlane32_swap); the score MFMAs start from minus the row's
+//                                      reference, which moves lazily; the causal mask is applied only
+//                                      on tiles that reach past the wave's first row
 //   block C   O^T += V^T . P^T         16 x v_mfma_f32_32x32x16_bf16; the accumulator layout of S^T is
 //                                      already the B-operand layout, V^T comes out of LDS through
 //                                      ds_read_b64_tr_b16 four MFMAs ahead; the exponent pipeline
-//                                      (exp2, sum and pack), skewed one slot per stage, rides in the slots
+//                                      (scale, exp2, sum and pack), skewed one slot per stage, rides in
+//                                      the slots (no scale instruction in the form that scales Q once)
 // In the steady part of the tile loop the per-tile bookkeeping is two scalar additions.
 //
 // What was measured on this part and shaped the kernel:
@@ -67,6 +67,7 @@
 // live registers per tile from every wave's instruction stream (-2 % run time on both benchmark shapes).
 #include "mops_common.h"
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 namespace mops {
@@ -127,7 +128,14 @@ __device__ __forceinline__ float max3(float a, float b, float c) { return __buil
 // workgroup barrier once this wave's LDS traffic is done and its loads into LDS have landed: what it publishes is the next tile
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// PRESCALE: Q is multiplied by softmax_scale * log2(e) when it is read and rounded back to bf16, so the scores leave the
+// MFMA as exponents (one VALU instruction per score less).  The rounding costs accuracy in proportion to the size of the
+// scores (an error of 2^-9 of a score in the exponent); without it the scale is applied in fp32, as the reference does.
+template <bool PRESCALE>
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const PrefillParams p) {
+  // the factor between a score as the MFMA delivers it and the base-2 exponent (the sign of a negative scale is moved into Q)
+  // (never exactly zero: a masked score is -inf, and -inf * 0 would be NaN where the probability has to be 0)
+  const float ec = PRESCALE ? 1.0f : fmaxf(fabsf(p.scale_log2), 1e-30f);
   // One array, so that the tile buffers start at the workgroup's LDS offset 0 whatever order the compiler lays shared
   // variables out in: a direct-to-LDS load takes its destination from M0 as a plain offset, and every tile offset here
   // stays below 64 KiB.  K[2] then V[2], then per wave the histogram of sequences by q tile count (compact launch).
@@ -487,11 +495,11 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     float alpha = 1.0f;
     const float m_old_safe = (m_run == -INFINITY) ? 0.f : m_run;
     const float m_abs = m_loc + m_old_safe;
-    const bool grow = m_abs > m_run + kLazyLog2;   // -inf reference: any finite maximum
+    const bool grow = m_abs * ec > m_run * ec + kLazyLog2;   // -inf reference: any finite maximum
     if (__any(grow)) {
       const float m_new = grow ? m_abs : m_run;
       const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha = __builtin_amdgcn_exp2f(m_run - m_new_safe);
+      alpha = __builtin_amdgcn_exp2f((m_run - m_new_safe) * ec);
       const float delta = m_new_safe - m_old_safe;   // 0 in lanes whose reference stays
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
@@ -506,8 +514,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     float f0[16], f1[16];   // per element pair q = 0..15 (elements 2q, 2q+1 of this lane's 32 scores): stage values
     auto stage_e = [&](int q) {
       const int tt = q >> 3, r = 2 * (q & 7);
-      f0[q] = __builtin_amdgcn_exp2f(s[tt][r]);
-      f1[q] = __builtin_amdgcn_exp2f(s[tt][r + 1]);
+      f0[q] = __builtin_amdgcn_exp2f(PRESCALE ? s[tt][r] : s[tt][r] * ec);
+      f1[q] = __builtin_amdgcn_exp2f(PRESCALE ? s[tt][r + 1] : s[tt][r + 1] * ec);
     };
     auto stage_p = [&](int q) {
       const int tt = q >> 3, r = 2 * (q & 7);
@@ -596,11 +604,11 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     float alpha = 1.0f;
     const float m_old_safe = (m_run == -INFINITY) ? 0.f : m_run;
     const float m_abs = m_loc + m_old_safe;
-    const bool grow = m_abs > m_run + kLazyLog2;
+    const bool grow = m_abs * ec > m_run * ec + kLazyLog2;
     if (__any(grow)) {
       const float m_new = grow ? m_abs : m_run;
       const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha = __builtin_amdgcn_exp2f(m_run - m_new_safe);
+      alpha = __builtin_amdgcn_exp2f((m_run - m_new_safe) * ec);
       const float delta = m_new_safe - m_old_safe;
 #pragma unroll
       for (int r = 0; r < 16; ++r) s0[r] -= delta;
@@ -612,8 +620,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     float ps0 = 0.f, ps1 = 0.f;
     float f0[8], f1[8];
     auto stage_e = [&](int q) {
-      f0[q] = __builtin_amdgcn_exp2f(s0[2 * q]);
-      f1[q] = __builtin_amdgcn_exp2f(s0[2 * q + 1]);
+      f0[q] = __builtin_amdgcn_exp2f(PRESCALE ? s0[2 * q] : s0[2 * q] * ec);
+      f1[q] = __builtin_amdgcn_exp2f(PRESCALE ? s0[2 * q + 1] : s0[2 * q + 1] * ec);
     };
     auto stage_p = [&](int q) {
       const int r = 2 * q;
@@ -668,12 +676,17 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const unsigned char* qt = lds + kPKTile + (wave & 1) * 8192 + (wave >> 1) * (2 * kPKTile);
 #pragma unroll
     for (int kb = 0; kb < 8; ++kb) {
-      // Q is scaled by softmax_scale * log2(e) here, once, and rounded back to bf16: the scores then come out of the
-      // MFMA in the exponent's units and the softmax spends no instruction on scaling them
+      // PRESCALE: Q is scaled by softmax_scale * log2(e) here, once, and rounded back to bf16: the scores then come out
+      // of the MFMA in the exponent's units and the softmax spends no instruction on scaling them
       u32x4 w = *reinterpret_cast<const u32x4*>(qt + rd_k[kb]);
+      if (PRESCALE) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        w[e] = pack_bf16x2(__builtin_bit_cast(float, w[e] << 16) * p.scale_log2, __builtin_bit_cast(float, w[e] & 0xffff0000u) * p.scale_log2);
+        for (int e = 0; e < 4; ++e)
+          w[e] = pack_bf16x2(__builtin_bit_cast(float, w[e] << 16) * p.scale_log2, __builtin_bit_cast(float, w[e] & 0xffff0000u) * p.scale_log2);
+      } else if (p.scale_log2 < 0.f) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] ^= 0x80008000u;   // -Q, exactly
+      }
       qb[kb] = __builtin_bit_cast(bf16x8, w);
     }
   }
@@ -786,6 +799,15 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   }
 }
 
+// MOPS_HIP_PREFILL_PRESCALE=1 selects the form that scales Q once (read at the first call)
+static bool prefill_prescale() {
+  static const bool on = [] {
+    const char* e = getenv("MOPS_HIP_PREFILL_PRESCALE");
+    return e && e[0] == '1';
+  }();
+  return on;
+}
+
 }  // namespace mops
 
 extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_stride,
@@ -859,6 +881,9 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   if (p.compact) pairs = pairs_bound;
   const int64_t grid = pairs * hq;
   if (grid > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
-  hipLaunchKernelGGL(varlen_prefill_kernel, dim3((unsigned)grid), dim3(kPThreads), 0, (hipStream_t)stream, p);
+  if (prefill_prescale())
+    hipLaunchKernelGGL(varlen_prefill_kernel<true>, dim3((unsigned)grid), dim3(kPThreads), 0, (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL(varlen_prefill_kernel<false>, dim3((unsigned)grid), dim3(kPThreads), 0, (hipStream_t)stream, p);
   return finish_launch();
 }

@@ -35,6 +35,58 @@ def test_prefill_matches_oracle(gpu, ops, lens, hq, hkv):
     assert_attention_close(got, _ref(ref, d), f"prefill lens={lens} {hq}:{hkv}")
 
 
+@pytest.mark.parametrize("scale,qmul", [(0.25, 1.0), (0.0, 1.0), (0.02, 30.0), (-0.0884, 1.0), (0.0884, 4.0), (1.0, 1.0)])
+def test_prefill_other_scales_and_large_scores(gpu, ops, scale, qmul):
+    """The scale is applied in fp32 to the fp32 scores, as the reference does (mops/triton/attention.py:83), so the error
+    does not grow with the size of the scores; the softmax reference is folded into the accumulator the score MFMAs start
+    from and moves only when a row maximum outgrows it by 2^8.  Scale 1 on N(0,1) data gives scores of +-40 in the
+    exponent's units (the reference moves again and again, probabilities collapse onto a few keys, outputs reach 4 and
+    their bf16 ulp 0.031), scale 0 a uniform softmax, a negative scale turns the order of the scores around."""
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefill_inputs([333, 64, 700], seed=17)
+    d["q"] = (d["q"].float() * qmul).to(torch.bfloat16)
+    d["scale"] = scale
+    got = _run(hip, d, gpu).float().cpu()
+    want = _ref(ref, d).float()
+    assert torch.isfinite(got).all()
+    diff = (got - want).abs()
+    assert diff.max().item() <= (4e-2 if scale == 1.0 else 2e-2), f"scale {scale}, q x {qmul}: max-abs {diff.max().item():.4g}"
+    assert diff.mean().item() <= 2e-3, f"scale {scale}, q x {qmul}: mean-abs {diff.mean().item():.4g}"
+
+
+def test_prefill_prescaled_q_form_meets_the_benchmark_tolerance(gpu):
+    """MOPS_HIP_PREFILL_PRESCALE=1 (read once per process, hence the child process) selects the form that multiplies Q by
+    scale * log2(e) once and rounds it back to bf16: faster, and within the benchmark's tolerance on the benchmark's
+    inputs, but its error grows with the size of the scores (at four times the benchmark's Q it leaves the tolerance)."""
+    import os, subprocess, sys
+    code = r'''
+import sys, torch
+sys.path.insert(0, ".")
+from nano_vllm_ninetoothed_amd import mops, workloads as W
+import oracle.mops_torch
+dev = torch.device("cuda:0")
+hip = mops.get_op("flash_attn_varlen_func", "hip"); ref = mops.get_op("flash_attn_varlen_func", "torch")
+for qmul in (1.0, 4.0):
+    d = W.prefill_inputs([333, 64, 700], seed=17)
+    d["q"] = (d["q"].float() * qmul).to(torch.bfloat16)
+    g = W.to_device(d, dev)
+    o = hip(g["q"], g["k"], g["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=g["cu_seqlens"], max_seqlen_k=d["max_seqlen"],
+            cu_seqlens_k=g["cu_seqlens"], softmax_scale=d["scale"], causal=True).cpu().float()
+    w = ref(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"], softmax_scale=d["scale"]).float()
+    e = (o - w).abs()
+    print(qmul, float(e.max()), float(e.mean()))
+'''
+    env = dict(os.environ, MOPS_HIP_PREFILL_PRESCALE="1")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=150)
+    assert out.returncode == 0, out.stderr[-2000:]
+    rows = [l.split() for l in out.stdout.strip().splitlines()[-2:]]
+    (q1, max1, mean1), (q4, max4, mean4) = [(float(a), float(b), float(c)) for a, b, c in rows]
+    assert (q1, q4) == (1.0, 4.0)
+    assert max1 <= 2e-2 and mean1 <= 2e-3, (max1, mean1)
+    assert mean4 > 2 * mean1, "the pre-scaled form is expected to lose accuracy as the scores grow"
+
+
 @pytest.mark.parametrize("nseq", [70, 200, 300])
 def test_prefill_many_ragged_sequences(gpu, ops, nseq):
     """Ragged batches launch workgroups for existing q tiles only (up to 256 sequences; sequence index found
