@@ -32,7 +32,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the default workload, calibrated against a 1 GiB copy
 DECODE_TRAFFIC_BYTES = 2497.6e6
 DECODE_TRAFFIC_SOURCE = "profiles/hbm_traffic_decode_prefill.txt (rocprofv3 --pmc, not measured by this run)"
-PREFILL_TRAFFIC_BYTES = {"prefill": 416.3e6, "prefill_long": 872.7e6}   # same source, same calibration
+PREFILL_TRAFFIC_BYTES = {"prefill": 409.4e6, "prefill_long": 871.3e6}   # same source, same calibration
 
 
 def parse_args():
