@@ -26,6 +26,9 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-Wall",
     "-Wno-unused-function",
+    # the direct-to-LDS loads are inline assembly that writes M0 and says so in its clobber list; the compiler warns
+    # that M0 is a reserved register (it never keeps a value there across statements, which is what the loads rely on)
+    "-Wno-inline-asm",
     # packed fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]

@@ -65,68 +65,12 @@
 // pos ^ 4 * (r & 3).  The K operand read (16 consecutive rows, one piece) and the transposing V read (4 rows x 2 x 32
 // bytes) then each cover all 64 banks once.  Against staging through registers this removes eight LDS stores and 32
 // live registers per tile from every wave's instruction stream (-2 % run time on both benchmark shapes).
-#include "mops_common.h"
+#include "prefill_common.h"
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
 namespace mops {
-
-constexpr int kPD = 128;            // head dim
-constexpr int kPBM = 128;           // q rows per workgroup
-constexpr int kPBN = 64;            // kv tokens per tile
-constexpr int kPThreads = 256;
-constexpr int kPRow = 256;          // bytes of one K or V row in LDS (128 bf16, no padding)
-constexpr int kPTile = kPBN * kPRow;        // 16384: a K or V tile
-constexpr int kPKChunk = 4 * kPRow;         // a tile is 16 chunks of 4 rows
-constexpr int kPKTile = kPTile;
-constexpr int kPAhead = 4;          // LDS operand reads run this many MFMAs ahead of use
-constexpr float kLazyLog2 = 8.0f;    // the softmax reference moves when a row maximum outgrows it by this much (base-2 exponent)
-constexpr int kPCompactChunks = 4;  // the compact launch handles up to 64 * 4 sequences
-
-struct PrefillParams {
-  const uint16_t* q;
-  const uint16_t* k;
-  const uint16_t* v;
-  uint16_t* out;
-  int64_t q_ts, k_ts, v_ts, o_ts;  // token strides (elements)
-  const int32_t* cu_seqlens;     // query side [batch+1]
-  const int32_t* cu_seqlens_k;   // key side [batch+1]; equal to cu_seqlens when there is no cached prefix
-  const int32_t* block_table;    // null: k/v are packed [total_k_tokens, hkv, 128]; else they are the paged caches
-  int64_t block_table_row_stride;
-  int block_size, num_blocks, max_blocks_per_seq;
-  int batch, total_tokens, total_k_tokens, m_tiles, hq, hkv, group;
-  int compact;   // workgroup ids enumerate only existing (q tile, sequence) pairs
-  float scale_log2;
-};
-
-// max / sum across the two 32-lane halves of the wave; every lane gets the result
-__device__ __forceinline__ float half_swap_max(float x) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float half_swap_sum(float x) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-// inclusive prefix sum over the 64 lanes of the wave (row shifts, then the two row broadcasts)
-__device__ __forceinline__ int wave_prefix_sum(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
-  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
-  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
-  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
-  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
-  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
-  return v;
-}
-
-// max of three; the compiler fuses the nested form into one v_max3_f32.  It has to stay a compiler-visible
-// operation: the wait states between an MFMA and the first VALU read of its result are inserted by the
-// compiler's hazard recognizer, which does not look inside inline assembly.
-__device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
-// workgroup barrier once this wave's LDS traffic is done and its loads into LDS have landed: what it publishes is the next tile
-__device__ __forceinline__ void tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // PRESCALE: Q is multiplied by softmax_scale * log2(e) when it is read and rounded back to bf16, so the scores leave the
 // MFMA as exponents (one VALU instruction per score less).  The rounding costs accuracy in proportion to the size of the
@@ -335,7 +279,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
     const char* src = base + voff;
     unsigned m0_tmp;
     asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %2\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 : "=&s"(m0_tmp) : "v"(src), "v"(lds_wave_base + lds_off) : "memory");
+                 : "=&s"(m0_tmp) : "v"(src), "v"(lds_wave_base + lds_off) : "memory", "m0");
   };
   // Steady-loop form: the tile's base address and the wave's LDS destination are scalar values (no vector instruction
   // forms an address or M0), the lane's offset from the tile base is one of eight precomputed registers.
@@ -344,7 +288,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
   // would make the statement safe for any operand and cost 1 % of the run time.
   auto to_lds_s = [&](uint64_t sbase, unsigned voff, unsigned lds_s) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 : : "v"(voff), "s"(sbase), "s"(lds_s) : "memory");
+                 : : "v"(voff), "s"(sbase), "s"(lds_s) : "memory", "m0");
   };
   // a wave-uniform value the compiler holds in a vector register, moved to a scalar one.  Wait states on both sides,
   // because the compiler's hazard bookkeeping does not see inside the statement: a v_readfirstlane right behind the
@@ -418,7 +362,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_kernel(const Pref
       const char* src_ = qbase + (int64_t)row * q_row_bytes + piece * 16;
       unsigned m0_tmp;
       asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %2\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                   : "=&s"(m0_tmp) : "v"(src_), "v"((unsigned)(uintptr_t)(lds_ptr_t)lds + q_lds + (unsigned)(1024 * i)) : "memory");
+                   : "=&s"(m0_tmp) : "v"(src_), "v"((unsigned)(uintptr_t)(lds_ptr_t)lds + q_lds + (unsigned)(1024 * i)) : "memory", "m0");
     }
   }
   f32x16 acc[4];
@@ -808,6 +752,14 @@ static bool prefill_prescale() {
   return on;
 }
 
+static bool prefill_force_rows() {
+  static const bool on = [] {
+    const char* e = getenv("MOPS_HIP_PREFILL_FORM");
+    return e && e[0] == 'r';
+  }();
+  return on;
+}
+
 }  // namespace mops
 
 extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_stride,
@@ -881,6 +833,13 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   if (p.compact) pairs = pairs_bound;
   const int64_t grid = pairs * hq;
   if (grid > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
+  // Grouped-query heads in pairs over the sequences' own keys take the form that packs two heads into a wave and keeps
+  // workgroups resident (varlen_prefill_pair.hip); everything else (cached prefix, paged caches, odd group sizes, very
+  // large batches, the form that scales Q once) stays here.  MOPS_HIP_PREFILL_FORM=rows forces this kernel.
+  if (!prefill_prescale() && !prefill_force_rows()) {
+    const int st = launch_prefill_pair(p, (hipStream_t)stream);
+    if (st != MOPS_HIP_EUNSUPPORTED) return st;
+  }
   if (prefill_prescale())
     hipLaunchKernelGGL(varlen_prefill_kernel<true>, dim3((unsigned)grid), dim3(kPThreads), 0, (hipStream_t)stream, p);
   else

@@ -1,0 +1,639 @@
+// Varlen (packed THD) causal prefill attention for gfx950, the form for grouped-query heads with an even group size and
+// keys that are the sequences' own tokens (no cached prefix): head_dim 128, bf16 MFMA for both products, fp32 online
+// softmax, K/V tiles staged through LDS.  The tile (blocks A, B, C, hand scheduled around the MFMAs) is the one of
+// varlen_prefill.hip; what differs is what a wave's 32 MFMA columns are and how work reaches a workgroup.
+//
+// Work decomposition
+//   item      = 64 query rows of one sequence x the two query heads 2u, 2u+1 (which share a kv head).  Wave w of the
+//               workgroup owns rows 16w .. 16w+15; MFMA column n of the wave is (head n >> 4, row n & 15).  Both heads read
+//               the same K/V tile from LDS, so the causal diagonal of an item is one 64 x 64 block instead of the 128 x 128
+//               of a 128-row item: half as many tile slots are spent on keys above the diagonal.
+//   launch    = resident workgroups (two per CU), each working through a list of items.  With 8 kv heads the workgroup id
+//               modulo 8 (the XCD it lands on) is the kv head it serves, so an XCD's L2 holds one kv head's K/V.  Items are
+//               ranked heaviest first (highest q tile first, then sequence).  A workgroup's first two items are fixed by its
+//               id, every further one is drawn from a counter in device memory two items ahead of its use, so that the
+//               draw and the rank -> item mapping are never waited for.
+//   hand-over = the K/V pipeline does not stop between items: the last tile of an item carries, in its MFMA slots, the
+//               direct-to-LDS loads of the next item's first K/V tile (into the tile buffers the last tile does not use) and
+//               the loads of the next item's Q operand (straight into the registers of the old one, which block A of the
+//               last tile has finished with).  What is left between two items is the epilogue of the old one.
+//   epilogue  = the wave's 32 columns x 128 outputs go through LDS (the buffers of the item's last tile, swizzled so that
+//               writes and reads cover all banks) and leave as whole 256-byte rows.
+#include "prefill_common.h"
+#include <atomic>
+#include <type_traits>
+
+namespace mops {
+
+constexpr int kPairRows = 64;          // q rows per item
+constexpr int kPairWaveRows = 16;      // q rows per wave (x 2 heads = 32 MFMA columns)
+constexpr int kPairMaxBatch = 512;     // sequences per launch (their offsets live in LDS)
+constexpr int kPairMaxTiles = 1024;    // q tiles per sequence (65536 tokens)
+constexpr int kPairSlots = 32;         // launches that may overlap on one device (one counter row each)
+
+// Item counters, one row per slot: [c] next ticket of class c (the workgroups with id % classes == c), [8] workgroups
+// that have finished.  The last workgroup to finish zeroes its row, so a row is all zeros between launches.
+__device__ unsigned g_pair_tickets[kPairSlots][16];
+
+struct PairLaunch {
+  int classes;          // 8 when there are 8 kv heads (class = kv head = XCD), else 1
+  int units_per_class;  // head pairs per class
+  int units_per_kv;     // head pairs per kv head (group / 2)
+  int members;          // workgroups per class
+  int q_tiles;          // bound on the q tiles (64 rows) of a sequence
+  int slot;             // counter row
+};
+
+// One 16-byte piece of the Q operand, loaded without the compiler knowing that the result arrives later: it then inserts
+// no wait of its own (which, placed in front of the first MFMAs that read the operand, would also wait for the tile
+// loads issued in between).  The operand is tied to its register on both sides, nothing reads it until the barrier at
+// the top of the next item's first tile, and that barrier waits for every load of the wave.
+template <int OFF>
+__device__ __forceinline__ void q_piece_async(bf16x8& dst, const char* ptr) {
+  asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "+v"(dst) : "v"(ptr), "n"(OFF) : "memory");
+}
+
+struct PairItem {
+  int valid, seq_begin, seq_len, q0, unit;
+};
+
+__global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const PrefillParams p, const PairLaunch L) {
+  // the factor between a score as the MFMA delivers it and the base-2 exponent (the sign of a negative scale is moved into Q)
+  // (never exactly zero: a masked score is -inf, and -inf * 0 would be NaN where the probability has to be 0)
+  const float ec = fmaxf(fabsf(p.scale_log2), 1e-30f);
+  // One array, so that the tile buffers start at the workgroup's LDS offset 0: a direct-to-LDS load takes its destination
+  // from M0 as a plain offset.  K[2] then V[2] (16 KiB each), then the tables of the rank -> item mapping.
+  constexpr int kTabCu = 0, kTabCnt = kPairMaxBatch + 4, kTabFrom = kTabCnt + kPairMaxBatch, kTabTicket = kTabFrom + kPairMaxTiles + 4;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPTile + (kTabTicket + 4) * 4];
+  int* const tab = reinterpret_cast<int*>(lds + 4 * kPTile);
+  int* const t_cu = tab + kTabCu;        // cu_seqlens [batch + 1]
+  int* const t_cnt = tab + kTabCnt;      // q tiles of sequence b
+  int* const t_from = tab + kTabFrom;    // (q tile, sequence) pairs whose q tile index is >= l, l = 0 .. q_tiles + 1
+  int* const t_tk = tab + kTabTicket;    // the ticket drawn during the current item
+  unsigned char* const lds_k = lds;
+  unsigned char* const lds_v = lds + 2 * kPKTile;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int n = lane & 31;    // MFMA column of the wave
+  const int jj = lane >> 5;   // half: k slice / row-quad selector
+  const int hsel = n >> 4;    // which of the unit's two heads the column belongs to
+  const int rloc = n & 15;    // its row inside the wave's 16 rows
+
+  // ---- tables of the rank -> item mapping (once per workgroup)
+  for (int i = tid; i <= p.batch; i += kPThreads) t_cu[i] = p.cu_seqlens[i];
+  __syncthreads();
+  for (int b = tid; b < p.batch; b += kPThreads) {
+    const int qs = t_cu[b];
+    const int len = min(t_cu[b + 1], p.total_tokens) - qs;
+    t_cnt[b] = (qs >= 0 && len > 0) ? min((len + kPairRows - 1) / kPairRows, L.q_tiles) : 0;
+  }
+  __syncthreads();
+  for (int l = tid; l <= L.q_tiles + 1; l += kPThreads) {
+    int s = 0;
+    if (l < L.q_tiles)
+      for (int b = 0; b < p.batch; ++b) s += max(0, t_cnt[b] - l);
+    t_from[l] = s;
+  }
+  __syncthreads();
+  const int cls = (int)blockIdx.x % L.classes;
+  const int member = (int)blockIdx.x / L.classes;
+  const int n_items = __builtin_amdgcn_readfirstlane(t_from[0]) * L.units_per_class;   // items of this class
+
+  // rank (within the class, heaviest first) -> item.  Every wave works it out for itself; all values are wave-uniform.
+  auto map_item = [&](int R) -> PairItem {
+    PairItem it = {0, 0, 0, 0, 0};
+    if (R >= n_items) return it;
+    const int pr = R / L.units_per_class;                       // rank of the (q tile, sequence) pair
+    const int unit = cls * L.units_per_class + R % L.units_per_class;
+    // the pair's q tile index m: the largest l with from[l] > pr; from[] is non-increasing, two levels of 64-way search
+    const int S = (L.q_tiles + 64) >> 6;
+    const int i1 = lane * S;
+    const int v1 = i1 <= L.q_tiles ? t_from[i1] : 0;
+    const unsigned long long m1 = __ballot(v1 > pr);
+    if (m1 == 0) return it;
+    int m = (63 - __builtin_clzll(m1)) * S;
+    if (S > 1) {
+      const int i2 = m + lane;
+      const int v2 = (lane < S && i2 <= L.q_tiles) ? t_from[i2] : 0;
+      const unsigned long long m2 = __ballot(v2 > pr);
+      m += 63 - __builtin_clzll(m2 | 1ull);
+    }
+    int r = pr - t_from[m + 1];   // rank among the sequences that have q tile m
+    int b = -1;
+    for (int j = 0; 64 * j < p.batch && b < 0; ++j) {
+      const int bb = lane + 64 * j;
+      const bool has = bb < p.batch && t_cnt[bb] > m;
+      const unsigned long long mask = __ballot(has);
+      const int c = __popcll(mask);
+      if (r < c) {
+        const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+        const unsigned long long hit = __ballot(has && before == r);
+        b = 64 * j + __builtin_ctzll(hit | (1ull << 63));
+      } else {
+        r -= c;
+      }
+    }
+    if (b < 0) return it;
+    const int seq_begin = t_cu[b];
+    const int seq_len = min(t_cu[b + 1], p.total_tokens) - seq_begin;
+    // q tiles are aligned to the END of the sequence: tile m covers rows [q0, q0 + 64) with q0 = len - 64 * (tiles - m), so
+    // the partial tile is the first one (rows below 0 do not exist), which looks at one K/V tile, and not the last one
+    const int seq_tiles = (seq_len + kPairRows - 1) / kPairRows;
+    it.valid = 1;
+    it.seq_begin = __builtin_amdgcn_readfirstlane(seq_begin);
+    it.seq_len = __builtin_amdgcn_readfirstlane(seq_len);
+    it.q0 = __builtin_amdgcn_readfirstlane(seq_len - (seq_tiles - m) * kPairRows);
+    it.unit = __builtin_amdgcn_readfirstlane(unit);
+    return it;
+  };
+
+  // ---- cooperative tile loads, HBM -> LDS without a stop in registers (global_load_lds_dwordx4: the 64 lanes of a wave
+  //      deposit 64 x 16 bytes at consecutive LDS addresses).  Instruction i of wave w brings rows 16i + 4w .. + 3 of the
+  //      tile: lane (rr = lane >> 4, pos = lane & 15) fills 16-byte position `pos` of row 16i + 4w + rr.  LDS rows are
+  //      unpadded; position pos of K row r holds piece pos ^ (r & 15), of V row r piece pos ^ 4 * (r & 3), so that the K
+  //      operand read and the transposing V read each cover all banks.  Rows past the end of the sequence read the
+  //      sequence's last row (finite data; their scores are masked, their probabilities zero).
+  const int ld_row = tid >> 4;     // 4 * wave + rr
+  const int ld_pos = tid & 15;
+  const unsigned k_row_bytes = (unsigned)(p.k_ts * 2), v_row_bytes = (unsigned)(p.v_ts * 2);
+  const unsigned kswz = (unsigned)((ld_pos ^ ld_row) << 4), vswz = (unsigned)((ld_pos ^ ((ld_row & 3) << 2)) << 4);
+  unsigned ko[4], vo[4];   // this lane's byte offsets of its pieces from a tile's base (the kv head is part of the base)
+  auto set_offsets = [&](int last) {   // last: last row of the tile that exists (63 for a whole tile)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned row = (unsigned)min(ld_row + 16 * i, last);
+      ko[i] = row * k_row_bytes + kswz;
+      vo[i] = row * v_row_bytes + vswz;
+    }
+  };
+  typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
+  // The tile's base address and the wave's LDS destination are scalar values, the lane's offset a vector register.
+  // M0 carries the wave's LDS destination; lane l deposits its 16 bytes at M0 + 16 * l.  Inline assembly on purpose:
+  // through the compiler's builtin every later LDS read waits for the load to land.
+  auto to_lds_s = [&](uint64_t sbase, unsigned voff, unsigned lds_s) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 : : "v"(voff), "s"(sbase), "s"(lds_s) : "memory", "m0");
+  };
+  // a wave-uniform value the compiler holds in a vector register, moved to a scalar one, with the wait states a
+  // v_readfirstlane needs behind the VALU write of its source and a memory instruction behind the write of a scalar base
+  auto to_scalar = [&](unsigned v) -> unsigned {
+    unsigned s_;
+    asm volatile("s_nop 1\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(s_) : "v"(v));
+    return s_;
+  };
+  const unsigned lds_s = to_scalar((unsigned)(uintptr_t)(lds_ptr_t)lds + ((unsigned)(tid >> 6) << 10));
+  // the eight loads of one tile in a burst (a wave that computes nothing on the tile)
+  auto loads_only = [&](uint64_t kbase, uint64_t vbase, unsigned lds_next) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) to_lds_s(kbase, ko[j], lds_next + (unsigned)(4 * kPKChunk * j));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) to_lds_s(vbase, vo[j], lds_next + (unsigned)(2 * kPKTile + 4 * kPKChunk * j));
+  };
+
+  // K operand read: lane (n, jj) reads piece jj + 2 * k8 of row n (+ 32): at position (jj + 2 * k8) ^ (n & 15)
+  int rd_k[8];
+#pragma unroll
+  for (int k8 = 0; k8 < 8; ++k8) rd_k[k8] = n * kPRow + (((jj + 2 * k8) ^ (n & 15)) << 4);
+  // transposing V read: 16-lane group (d half, jj); lane addresses token row 4 * jj + rr2 of a 4-row set and 8 bytes of
+  // the group's 32-byte window; the 64-byte block dt of the row sits at block dt ^ rr2
+  int rd_v[4];
+  {
+    const int rr2 = (lane >> 2) & 3;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+      rd_v[dt] = (4 * jj + rr2) * kPRow + (((lane >> 4) & 1) << 5) + ((lane & 3) << 3) + 64 * (dt ^ rr2);
+  }
+
+  // ---- per-item state
+  bf16x8 qb[8];   // Q^T as B operand: lane (n, jj) holds Q[row][head][16*kb + 8*jj .. +8) for kb = 0..7
+  f32x16 acc[4];
+  f32x16 s_init;  // the accumulator every score product starts from: minus the softmax reference
+  float m_run, l_run;
+  const int64_t q_row_bytes = p.q_ts * 2;
+  // address of this lane's first Q piece of an item; rows outside the sequence take a copy of a valid row (columns are
+  // independent and theirs are never stored)
+  auto q_address = [&](const PairItem& it) -> const char* {
+    const int row = min(max(it.q0 + kPairWaveRows * wave + rloc, 0), it.seq_len - 1);
+    return reinterpret_cast<const char*>(p.q) + (int64_t)(it.seq_begin + row) * q_row_bytes + (int64_t)((2 * it.unit + hsel) * kPD + 8 * jj) * 2;
+  };
+  auto q_load = [&](int kb, const char* ptr) {
+    switch (kb) {
+      case 0: q_piece_async<0>(qb[0], ptr); break;
+      case 1: q_piece_async<32>(qb[1], ptr); break;
+      case 2: q_piece_async<64>(qb[2], ptr); break;
+      case 3: q_piece_async<96>(qb[3], ptr); break;
+      case 4: q_piece_async<128>(qb[4], ptr); break;
+      case 5: q_piece_async<160>(qb[5], ptr); break;
+      case 6: q_piece_async<192>(qb[6], ptr); break;
+      default: q_piece_async<224>(qb[7], ptr); break;
+    }
+  };
+  auto kv_base = [&](const PairItem& it, const uint16_t* base, int64_t ts) -> uint64_t {
+    const int g = it.unit / L.units_per_kv;
+    return reinterpret_cast<uint64_t>(base) + (uint64_t)(((int64_t)it.seq_begin * ts + (int64_t)g * kPD) * 2);
+  };
+
+  // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
+  // scheduling fence are what the wave issues while that MFMA runs.
+  //   block A: S^T = K . Q^T, the eight direct-to-LDS loads of the next tile ride in its slots
+  //   block B: row max, whether the reference has to move, the first ten exponentials
+  //   block C: O^T += V^T . P^T, the remaining exponentials, the row sums and the bf16 packing ride in its slots; on an
+  //            item's last tile (`last`) also the eight loads of the next item's Q operand, into qb, which block A is done with
+  // `horizon`: last key (sequence-relative) this lane's row may see; only read on the masked variant.
+  auto tile_compute = [&](int tile, int buf, uint64_t kbase, uint64_t vbase, auto masked, auto last, int horizon, const char* qnext) {
+    const unsigned lds_next = lds_s + (unsigned)((buf ^ 1) * kPKTile);
+    f32x16 s[2];
+    {
+      const unsigned char* kt = lds_k + buf * kPKTile;
+      u32x4 ka[16];
+      auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + rd_k[i >> 1] + (i & 1) * 32 * kPRow); };
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i >> 1], i < 2 ? s_init : s[i & 1], 0, 0, 0);
+        if (i + kPAhead < 16) rd(i + kPAhead);
+        if (i & 1) {
+          const int j = i >> 1;
+          if (j < 4) to_lds_s(kbase, ko[j], lds_next + (unsigned)(4 * kPKChunk * j));
+          else to_lds_s(vbase, vo[j - 4], lds_next + (unsigned)(2 * kPKTile + 4 * kPKChunk * (j - 4)));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    // block B
+    if (decltype(masked)::value) {
+      const int j0 = tile * kPBN;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = j0 + 32 * tt + 8 * (r >> 2) + 4 * jj + (r & 3);
+          s[tt][r] = key <= horizon ? s[tt][r] : -INFINITY;
+        }
+    }
+    // A wave issues in order and a dependent VALU instruction waits ~20 cycles for its operand, so the
+    // softmax is written for instruction-level parallelism: four max chains, and the exponent pipeline
+    // E (exp2) -> P (row sum, bf16 pack) is skewed by one MFMA slot per stage.
+    float mx[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) mx[c] = max3(s[c >> 1][8 * (c & 1)], s[c >> 1][8 * (c & 1) + 1], s[c >> 1][8 * (c & 1) + 2]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) mx[c] = max3(mx[c], s[c >> 1][8 * (c & 1) + 3], s[c >> 1][8 * (c & 1) + 4]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) mx[c] = max3(mx[c], s[c >> 1][8 * (c & 1) + 5], s[c >> 1][8 * (c & 1) + 6]);
+    const float m01 = max3(mx[0], mx[1], s[0][7]), m23 = max3(mx[2], mx[3], s[0][15]);
+    const float m_loc = half_swap_max(max3(m01, m23, fmaxf(s[1][7], s[1][15])));
+    // m_loc is relative to the reference the scores were computed against.  The reference only moves when a row's
+    // maximum outgrows it by kLazyLog2 (probabilities then reach at most 2^kLazyLog2, harmless in bf16 and in the fp32
+    // sums; the final division by the row sum is exact for any reference).
+    float alpha = 1.0f;
+    const float m_old_safe = (m_run == -INFINITY) ? 0.f : m_run;
+    const float m_abs = m_loc + m_old_safe;
+    const bool grow = m_abs * ec > m_run * ec + kLazyLog2;   // -inf reference: any finite maximum
+    if (__any(grow)) {
+      const float m_new = grow ? m_abs : m_run;
+      const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha = __builtin_amdgcn_exp2f((m_run - m_new_safe) * ec);
+      const float delta = m_new_safe - m_old_safe;   // 0 in lanes whose reference stays
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[tt][r] -= delta;
+      m_run = m_new;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_init[r] = -m_new_safe;
+    }
+    u32x4 pw[4];   // P^T as B operand for the four 16-token k blocks
+    float ps0 = 0.f, ps1 = 0.f;
+    float f0[16], f1[16];
+    auto stage_e = [&](int q) {
+      const int tt = q >> 3, r = 2 * (q & 7);
+      f0[q] = __builtin_amdgcn_exp2f(s[tt][r] * ec);
+      f1[q] = __builtin_amdgcn_exp2f(s[tt][r + 1] * ec);
+    };
+    auto stage_p = [&](int q) {
+      const int tt = q >> 3, r = 2 * (q & 7);
+      if (q & 1) ps1 += f0[q] + f1[q]; else ps0 += f0[q] + f1[q];
+      pw[2 * tt + (r >> 3)][(r & 7) >> 1] = pack_bf16x2(f0[q], f1[q]);
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < 5; ++q) stage_e(q);
+    __builtin_amdgcn_sched_barrier(0);
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_p(q);
+    // block C
+    {
+      const unsigned char* vt = lds_v + buf * kPTile;
+      s16x4 vlo[16], vhi[16];
+      auto rd = [&](int i) {
+        const int kb2 = i >> 2, dt = i & 3;
+        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + 16 * kb2 * kPRow));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + (16 * kb2 + 8) * kPRow));
+      };
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
+        if (i + kPAhead < 16) rd(i + kPAhead);
+        // slot i finishes pair i + 4 (needed from slot 4 * ((i + 4) / 4) on) and exponentiates pair i + 5
+        if (i + 4 < 16) stage_p(i + 4);
+        if (i + 5 < 16) stage_e(i + 5);
+        if (decltype(last)::value && (i & 1)) q_load(i >> 1, qnext);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    l_run = l_run * alpha + (ps0 + ps1);
+  };
+
+  // The same for a tile of which no row of this wave sees more than the first 32 keys: the fully masked half is neither
+  // multiplied nor exponentiated.  Eight MFMAs per block.
+  auto tile_compute_half = [&](int tile, int buf, uint64_t kbase, uint64_t vbase, auto last, int horizon, const char* qnext) {
+    const unsigned lds_next = lds_s + (unsigned)((buf ^ 1) * kPKTile);
+    f32x16 s0;
+    {
+      const unsigned char* kt = lds_k + buf * kPKTile;
+      u32x4 ka[8];
+      auto rd = [&](int i) { ka[i] = *reinterpret_cast<const u32x4*>(kt + rd_k[i]); };
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qb[i], i == 0 ? s_init : s0, 0, 0, 0);
+        if (i + kPAhead < 8) rd(i + kPAhead);
+        if (i < 4) to_lds_s(kbase, ko[i], lds_next + (unsigned)(4 * kPKChunk * i));
+        else to_lds_s(vbase, vo[i - 4], lds_next + (unsigned)(2 * kPKTile + 4 * kPKChunk * (i - 4)));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    {
+      const int j0 = tile * kPBN;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = j0 + 8 * (r >> 2) + 4 * jj + (r & 3);
+        s0[r] = key <= horizon ? s0[r] : -INFINITY;
+      }
+    }
+    float mx[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mx[c] = max3(s0[8 * c], s0[8 * c + 1], s0[8 * c + 2]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mx[c] = max3(mx[c], s0[8 * c + 3], s0[8 * c + 4]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mx[c] = max3(mx[c], s0[8 * c + 5], s0[8 * c + 6]);
+    const float m_loc = half_swap_max(max3(mx[0], mx[1], fmaxf(s0[7], s0[15])));
+    float alpha = 1.0f;
+    const float m_old_safe = (m_run == -INFINITY) ? 0.f : m_run;
+    const float m_abs = m_loc + m_old_safe;
+    const bool grow = m_abs * ec > m_run * ec + kLazyLog2;
+    if (__any(grow)) {
+      const float m_new = grow ? m_abs : m_run;
+      const float m_new_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha = __builtin_amdgcn_exp2f((m_run - m_new_safe) * ec);
+      const float delta = m_new_safe - m_old_safe;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s0[r] -= delta;
+      m_run = m_new;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_init[r] = -m_new_safe;
+    }
+    u32x4 pw[2];
+    float ps0 = 0.f, ps1 = 0.f;
+    float f0[8], f1[8];
+    auto stage_e = [&](int q) {
+      f0[q] = __builtin_amdgcn_exp2f(s0[2 * q] * ec);
+      f1[q] = __builtin_amdgcn_exp2f(s0[2 * q + 1] * ec);
+    };
+    auto stage_p = [&](int q) {
+      const int r = 2 * q;
+      if (q & 1) ps1 += f0[q] + f1[q]; else ps0 += f0[q] + f1[q];
+      pw[r >> 3][(r & 7) >> 1] = pack_bf16x2(f0[q], f1[q]);
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < 5; ++q) stage_e(q);
+    __builtin_amdgcn_sched_barrier(0);
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_p(q);
+    {
+      const unsigned char* vt = lds_v + buf * kPTile;
+      s16x4 vlo[8], vhi[8];
+      auto rd = [&](int i) {
+        const int kb2 = i >> 2, dt = i & 3;
+        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + 16 * kb2 * kPRow));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vt + rd_v[dt] + (16 * kb2 + 8) * kPRow));
+      };
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      for (int i0 = 0; i0 < kPAhead; ++i0) rd(i0);
+      __builtin_amdgcn_s_setprio(1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const s16x8 a8 = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, pw[i >> 2]), acc[i & 3], 0, 0, 0);
+        if (i + kPAhead < 8) rd(i + kPAhead);
+        if (i + 4 < 8) stage_p(i + 4);
+        if (i + 5 < 8) stage_e(i + 5);
+        if (decltype(last)::value) q_load(i, qnext);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    l_run = l_run * alpha + (ps0 + ps1);
+  };
+
+  // ---- the workgroup's first two items; the first one's Q operand and first K/V tile
+  PairItem cur = map_item(member);
+  PairItem nxt = map_item(member + L.members);
+  unsigned* const tickets = g_pair_tickets[L.slot];
+  const uint64_t kstep = (uint64_t)kPBN * (uint64_t)p.k_ts * 2u, vstep = (uint64_t)kPBN * (uint64_t)p.v_ts * 2u;
+  int clamp = 63;     // the last-row clamp ko / vo are set for
+  int buf = 0;        // tile buffer pair the tile about to be computed sits in
+  if (cur.valid) {
+    clamp = min(63, cur.seq_len - 1);
+    set_offsets(clamp);
+    loads_only(kv_base(cur, p.k, p.k_ts), kv_base(cur, p.v, p.v_ts), lds_s);
+    const char* qa = q_address(cur);
+#pragma unroll
+    for (int kb = 0; kb < 8; ++kb) q_load(kb, qa);
+  }
+
+  unsigned tk = 0;   // thread 0: the ticket in flight
+  // The barrier at the top of a tile, followed by a use of the ticket register: the barrier has waited for every memory
+  // operation of the wave, the atomic included, and the (empty) use tells the compiler so; otherwise it would wait for the
+  // atomic's result where the register is next written, at the top of the next item, and for everything issued before it.
+  auto item_barrier = [&]() {
+    tile_barrier();
+    asm volatile("" : : "v"(tk));
+  };
+  while (cur.valid) {
+    if (p.scale_log2 < 0.f) {   // the sign of a negative scale moves into Q; the operand has to have arrived for that
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(qb[0]), "+v"(qb[1]), "+v"(qb[2]), "+v"(qb[3]), "+v"(qb[4]), "+v"(qb[5]), "+v"(qb[6]), "+v"(qb[7]));
+#pragma unroll
+      for (int kb = 0; kb < 8; ++kb) qb[kb] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, qb[kb]) ^ 0x80008000u);   // -Q, exactly
+    }
+    // The ticket of the item after next; thread 0 parks it in LDS behind the item's first barrier.  A wrapping increment
+    // and not an addition: the compiler turns a uniform atomic addition into one lane's addition plus a broadcast of the
+    // result, which would wait for the result right here.
+    if (tid == 0 && nxt.valid) tk = atomicInc(&tickets[cls], 0xffffffffu);
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_init[r] = 0.f;
+    m_run = -INFINITY;
+    l_run = 0.f;
+
+    const int ntiles = (cur.q0 + kPairRows + kPBN - 1) / kPBN;      // K/V tiles the item looks at (keys 0 .. q0 + 63)
+    const int wave_row0 = cur.q0 + kPairWaveRows * wave;           // first q row (sequence-relative) of this wave
+    const int my_row = wave_row0 + rloc;
+    // tiles this wave has to look at, and those of them that lie wholly below its first row's diagonal
+    const int my_tiles = wave_row0 + kPairWaveRows - 1 >= 0 ? min(ntiles, (wave_row0 + kPairWaveRows - 1) / kPBN + 1) : 0;
+    const int unmasked = wave_row0 >= 0 ? (wave_row0 + 1) / kPBN : 0;
+    uint64_t kbase = kv_base(cur, p.k, p.k_ts), vbase = kv_base(cur, p.v, p.v_ts);   // base of the tile after the one being computed
+    int tile = 0;
+    for (; tile < ntiles - 1; ++tile) {
+      item_barrier();
+      if (tile == 0 && tid == 0) t_tk[0] = (int)tk;
+      kbase += kstep;
+      vbase += vstep;
+      // the successor is a tile of this item; only the item's last tile can reach past the end of the sequence
+      const int want = min(63, cur.seq_len - 1 - (tile + 1) * kPBN);
+      if (want != clamp) {
+        clamp = want;
+        set_offsets(clamp);
+      }
+      if (tile >= my_tiles) loads_only(kbase, vbase, lds_s + (unsigned)((buf ^ 1) * kPKTile));
+      else if (tile < unmasked) tile_compute(tile, buf, kbase, vbase, std::false_type{}, std::false_type{}, 0, nullptr);
+      else if (wave_row0 + kPairWaveRows - 1 < tile * kPBN + 32) tile_compute_half(tile, buf, kbase, vbase, std::false_type{}, my_row, nullptr);
+      else tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::false_type{}, my_row, nullptr);
+      buf ^= 1;
+    }
+    // the item's last tile: its successor is the next item's first tile, and the next item's Q operand comes with it.
+    // Without a next item the loads are repeated on this item's own first tile and rows (harmless, never read).
+    {
+      item_barrier();
+      if (tile == 0 && tid == 0) t_tk[0] = (int)tk;
+      const PairItem& to = nxt.valid ? nxt : cur;
+      kbase = kv_base(to, p.k, p.k_ts);
+      vbase = kv_base(to, p.v, p.v_ts);
+      const int want = min(63, to.seq_len - 1);
+      if (want != clamp) {
+        clamp = want;
+        set_offsets(clamp);
+      }
+      const char* qnext = q_address(to);
+      if (tile >= my_tiles) {
+        loads_only(kbase, vbase, lds_s + (unsigned)((buf ^ 1) * kPKTile));
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) q_load(kb, qnext);
+      } else if (wave_row0 + kPairWaveRows - 1 < tile * kPBN + 32) {
+        tile_compute_half(tile, buf, kbase, vbase, std::true_type{}, my_row, qnext);
+      } else {
+        tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::true_type{}, my_row, qnext);
+      }
+    }
+    item_barrier();   // every wave is done with the last tile: its buffer pair is free for the epilogue
+
+    // ---- epilogue.  A lane holds 8-byte pieces of its own column, which would make every store instruction touch 64
+    //      cache lines; the wave's 32 columns x 256 bytes go through LDS instead (the wave's quarter of the last tile's
+    //      buffer pair) and leave as whole 256-byte rows, four per store instruction.  Column n's 16-byte piece P sits at
+    //      position P ^ (n & 15) and its two halves are exchanged for the second head's columns: the 32 lanes of a write
+    //      pass and the 16 lanes of a read pass then each cover all banks.
+    l_run = half_swap_sum(l_run);
+    {
+      const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+      unsigned char* const stage = lds + (wave < 2 ? buf * kPKTile : 2 * kPKTile + buf * kPTile) + (wave & 1) * 8192;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          u32x2 w;
+          w[0] = pack_bf16x2(acc[dt][4 * rq] * inv, acc[dt][4 * rq + 1] * inv);
+          w[1] = pack_bf16x2(acc[dt][4 * rq + 2] * inv, acc[dt][4 * rq + 3] * inv);
+          *reinterpret_cast<u32x2*>(stage + n * kPRow + (((4 * dt + rq) ^ rloc) << 4) + ((jj ^ hsel) << 3)) = w;
+        }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes, read back by other lanes
+      int piece = lane & 15, c4 = lane >> 4;
+      // opaque to the compiler on purpose: otherwise it works the addresses of the eight reads and stores out once, before
+      // the item loop, and keeps them in registers it does not have (they were spilled, and reloading them here made every
+      // item wait for its own output stores)
+      asm volatile("" : "+v"(piece), "+v"(c4));
+      uint16_t* const obase = p.out + (int64_t)(cur.seq_begin + wave_row0) * p.o_ts + (int64_t)(2 * cur.unit) * kPD + 8 * piece;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int col = 4 * i + c4;           // column of the wave: head i >> 2, row col & 15
+        const int row = col & 15;
+        u32x4 w = *reinterpret_cast<const u32x4*>(stage + col * kPRow + ((piece ^ row) << 4));
+        if (i >= 4) w = u32x4{w[2], w[3], w[0], w[1]};
+        // written once and not read again here: a streaming store leaves less for the write-back at the end of the kernel
+        if (wave_row0 + row >= 0) __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts + (i >> 2) * kPD));
+      }
+    }
+    buf ^= 1;
+    // ---- the item after next, from the ticket drawn at the top
+    PairItem after = {0, 0, 0, 0, 0};
+    if (nxt.valid) after = map_item(2 * L.members + __builtin_amdgcn_readfirstlane(t_tk[0]));
+    cur = nxt;
+    nxt = after;
+  }
+
+  // ---- the last workgroup to finish clears the counters for the next launch that uses this row
+  if (tid == 0) {
+    const unsigned done = atomicAdd(&tickets[8], 1u);
+    if (done == gridDim.x - 1) {
+      for (int c = 0; c < 9; ++c) __hip_atomic_store(&tickets[c], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+int launch_prefill_pair(const PrefillParams& p, hipStream_t stream) {
+  if (p.block_table != nullptr || p.cu_seqlens_k != p.cu_seqlens || p.total_k_tokens != p.total_tokens) return MOPS_HIP_EUNSUPPORTED;
+  if (p.group < 2 || (p.group & 1) || p.batch > kPairMaxBatch) return MOPS_HIP_EUNSUPPORTED;
+  PairLaunch L;
+  // m_tiles counts 128-row tiles of the longest sequence; twice as many 64-row tiles bound it here
+  L.q_tiles = 2 * p.m_tiles;
+  if (L.q_tiles > kPairMaxTiles) return MOPS_HIP_EUNSUPPORTED;
+  const int units = p.hq / 2;
+  L.classes = p.hkv == 8 ? 8 : 1;
+  L.units_per_class = units / L.classes;
+  L.units_per_kv = p.group / 2;
+  static std::atomic<int> cu_count[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MOPS_HIP_EUNSUPPORTED;
+  int cus = cu_count[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return MOPS_HIP_EUNSUPPORTED;
+    cu_count[dev].store(cus, std::memory_order_relaxed);
+  }
+  // two resident workgroups per CU; fewer when the launch cannot hold that many items
+  const int64_t items_bound = ((int64_t)p.total_tokens / kPairRows + p.batch) * L.units_per_class;
+  L.members = (int)std::min<int64_t>(items_bound, std::max(1, 2 * cus / L.classes));
+  static std::atomic<unsigned> next_slot{0};
+  L.slot = (int)(next_slot.fetch_add(1, std::memory_order_relaxed) % kPairSlots);
+  hipLaunchKernelGGL(varlen_prefill_pair_kernel, dim3((unsigned)(L.members * L.classes)), dim3(kPThreads), 0, stream, p, L);
+  return finish_launch();
+}
+
+}  // namespace mops
