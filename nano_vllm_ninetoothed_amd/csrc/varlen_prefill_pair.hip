@@ -11,8 +11,8 @@
 //   launch    = resident workgroups (two per CU), each working through a list of items.  With 8 kv heads the workgroup id
 //               modulo 8 (the XCD it lands on) is the kv head it serves, so an XCD's L2 holds one kv head's K/V.  Items are
 //               ranked heaviest first (highest q tile first, then sequence).  A workgroup's first two items are fixed by its
-//               id, every further one is drawn from a counter in device memory two items ahead of its use, so that the
-//               draw and the rank -> item mapping are never waited for.
+//               id; every further one is drawn from a counter in device memory at the top of the item before it, and the
+//               ticket has arrived by that item's last tile (an item of one tile waits for it).
 //   hand-over = the K/V pipeline does not stop between items: the last tile of an item carries, in its MFMA slots, the
 //               direct-to-LDS loads of the next item's first K/V tile (into the tile buffers the last tile does not use) and
 //               the loads of the next item's Q operand (straight into the registers of the old one, which block A of the
@@ -463,8 +463,10 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   };
 
   // ---- the workgroup's first two items; the first one's Q operand and first K/V tile
+  //      (ranks j and 2 * members - 1 - j: the heaviest first item goes with the lightest second one)
   PairItem cur = map_item(member);
-  PairItem nxt = map_item(member + L.members);
+  PairItem nxt = map_item(2 * L.members - 1 - member);
+  bool draw = false;   // whether the item after the current one is drawn from the counter (every item but the first two)
   unsigned* const tickets = g_pair_tickets[L.slot];
   const uint64_t kstep = (uint64_t)kPBN * (uint64_t)p.k_ts * 2u, vstep = (uint64_t)kPBN * (uint64_t)p.v_ts * 2u;
   int clamp = 63;     // the last-row clamp ko / vo are set for
@@ -486,6 +488,11 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     tile_barrier();
     asm volatile("" : : "v"(tk));
   };
+  // Whether the wave's last eight vector-memory instructions before the top of this item were the eight output stores of
+  // the previous item (every row of the wave existed; else the stores are predicated and may be skipped).  The item's first
+  // barrier then waits for everything but those stores: the loads of the item's first tile and of its Q operand are older,
+  // memory operations complete in order, and the acknowledgement of a store is nothing the item needs.
+  bool stores8 = false;
   while (cur.valid) {
     if (p.scale_log2 < 0.f) {   // the sign of a negative scale moves into Q; the operand has to have arrived for that
       asm volatile("s_waitcnt vmcnt(0)" : "+v"(qb[0]), "+v"(qb[1]), "+v"(qb[2]), "+v"(qb[3]), "+v"(qb[4]), "+v"(qb[5]), "+v"(qb[6]), "+v"(qb[7]));
@@ -495,7 +502,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     // The ticket of the item after next; thread 0 parks it in LDS behind the item's first barrier.  A wrapping increment
     // and not an addition: the compiler turns a uniform atomic addition into one lane's addition plus a broadcast of the
     // result, which would wait for the result right here.
-    if (tid == 0 && nxt.valid) tk = atomicInc(&tickets[cls], 0xffffffffu);
+    if (tid == 0 && draw) tk = atomicInc(&tickets[cls], 0xffffffffu);
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -512,10 +519,14 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     const int my_tiles = wave_row0 + kPairWaveRows - 1 >= 0 ? min(ntiles, (wave_row0 + kPairWaveRows - 1) / kPBN + 1) : 0;
     const int unmasked = wave_row0 >= 0 ? (wave_row0 + 1) / kPBN : 0;
     uint64_t kbase = kv_base(cur, p.k, p.k_ts), vbase = kv_base(cur, p.v, p.v_ts);   // base of the tile after the one being computed
+    // The item's first barrier.  (Thread 0's wave has one more operation in flight, the draw; eight may stay in flight there
+    // too, which then makes it wait for one store.)  The ticket goes to LDS behind a barrier that has waited for the draw:
+    // the second one, or, for items of one or two tiles, here, where the compiler puts the wait in front of the write.
+    if (stores8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else tile_barrier();
+    if (ntiles <= 2 && tid == 0 && draw) t_tk[0] = (int)tk;
     int tile = 0;
     for (; tile < ntiles - 1; ++tile) {
-      item_barrier();
-      if (tile == 0 && tid == 0) t_tk[0] = (int)tk;
       kbase += kstep;
       vbase += vstep;
       // the successor is a tile of this item; only the item's last tile can reach past the end of the sequence
@@ -529,12 +540,18 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
       else if (wave_row0 + kPairWaveRows - 1 < tile * kPBN + 32) tile_compute_half(tile, buf, kbase, vbase, std::false_type{}, my_row, nullptr);
       else tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::false_type{}, my_row, nullptr);
       buf ^= 1;
+      item_barrier();   // the top of the next tile
+      if (tile == 0 && ntiles > 2 && tid == 0 && draw) t_tk[0] = (int)tk;
     }
     // the item's last tile: its successor is the next item's first tile, and the next item's Q operand comes with it.
     // Without a next item the loads are repeated on this item's own first tile and rows (harmless, never read).
     {
-      item_barrier();
-      if (tile == 0 && tid == 0) t_tk[0] = (int)tk;
+      if (draw) {
+        // The ticket drawn at the top of the item went to LDS one barrier ago at the latest; an item of a single tile has
+        // come through one barrier only and holds another one here.
+        if (ntiles == 1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        nxt = map_item(2 * L.members + __builtin_amdgcn_readfirstlane(t_tk[0]));
+      }
       const PairItem& to = nxt.valid ? nxt : cur;
       kbase = kv_base(to, p.k, p.k_ts);
       vbase = kv_base(to, p.v, p.v_ts);
@@ -581,22 +598,27 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
       // item wait for its own output stores)
       asm volatile("" : "+v"(piece), "+v"(c4));
       uint16_t* const obase = p.out + (int64_t)(cur.seq_begin + wave_row0) * p.o_ts + (int64_t)(2 * cur.unit) * kPD + 8 * piece;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      auto out_piece = [&](int i, auto all_rows) {
         const int col = 4 * i + c4;           // column of the wave: head i >> 2, row col & 15
         const int row = col & 15;
         u32x4 w = *reinterpret_cast<const u32x4*>(stage + col * kPRow + ((piece ^ row) << 4));
         if (i >= 4) w = u32x4{w[2], w[3], w[0], w[1]};
         // written once and not read again here: a streaming store leaves less for the write-back at the end of the kernel
-        if (wave_row0 + row >= 0) __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts + (i >> 2) * kPD));
+        if (decltype(all_rows)::value || wave_row0 + row >= 0)
+          __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts + (i >> 2) * kPD));
+      };
+      stores8 = __builtin_amdgcn_readfirstlane(wave_row0) >= 0;   // rows below 0 only exist in a sequence's first q tile
+      if (stores8) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out_piece(i, std::true_type{});
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out_piece(i, std::false_type{});
       }
     }
     buf ^= 1;
-    // ---- the item after next, from the ticket drawn at the top
-    PairItem after = {0, 0, 0, 0, 0};
-    if (nxt.valid) after = map_item(2 * L.members + __builtin_amdgcn_readfirstlane(t_tk[0]));
     cur = nxt;
-    nxt = after;
+    draw = true;
   }
 
   // ---- the last workgroup to finish clears the counters for the next launch that uses this row
