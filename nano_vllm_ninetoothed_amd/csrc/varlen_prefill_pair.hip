@@ -29,7 +29,7 @@ constexpr int kPairRows = 64;          // q rows per item
 constexpr int kPairWaveRows = 16;      // q rows per wave (x 2 heads = 32 MFMA columns)
 constexpr int kPairMaxBatch = 512;     // sequences per launch (their offsets live in LDS)
 constexpr int kPairMaxTiles = 1024;    // q tiles per sequence (65536 tokens)
-constexpr int kPairSlots = 32;         // launches that may overlap on one device (one counter row each)
+constexpr int kPairSlots = 128;        // launches that may overlap on one device (one counter row each)
 
 // Item counters, one row per slot: [c] next ticket of class c (the workgroups with id % classes == c), [8] workgroups
 // that have finished.  The last workgroup to finish zeroes its row, so a row is all zeros between launches.
@@ -97,12 +97,13 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     t_from[l] = s;
   }
   __syncthreads();
-  const int cls = (int)blockIdx.x % L.classes;
+  const int home = (int)blockIdx.x % L.classes;   // the class this workgroup serves first
   const int member = (int)blockIdx.x / L.classes;
-  const int n_items = __builtin_amdgcn_readfirstlane(t_from[0]) * L.units_per_class;   // items of this class
+  const int n_items = __builtin_amdgcn_readfirstlane(t_from[0]) * L.units_per_class;   // items of a class (the same for all)
+  if (tid == 0) t_tk[2] = home;
 
   // rank (within the class, heaviest first) -> item.  Every wave works it out for itself; all values are wave-uniform.
-  auto map_item = [&](int R) -> PairItem {
+  auto map_item = [&](int cls, int R) -> PairItem {
     PairItem it = {0, 0, 0, 0, 0};
     if (R >= n_items) return it;
     const int pr = R / L.units_per_class;                       // rank of the (q tile, sequence) pair
@@ -122,8 +123,10 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     }
     int r = pr - t_from[m + 1];   // rank among the sequences that have q tile m
     int b = -1;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));   // opaque: keeps the compiler from holding this loop's LDS addresses in registers for the whole kernel
     for (int j = 0; 64 * j < p.batch && b < 0; ++j) {
-      const int bb = lane + 64 * j;
+      const int bb = ln + 64 * j;
       const bool has = bb < p.batch && t_cnt[bb] > m;
       const unsigned long long mask = __ballot(has);
       const int c = __popcll(mask);
@@ -464,8 +467,8 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
 
   // ---- the workgroup's first two items; the first one's Q operand and first K/V tile
   //      (ranks j and 2 * members - 1 - j: the heaviest first item goes with the lightest second one)
-  PairItem cur = map_item(member);
-  PairItem nxt = map_item(2 * L.members - 1 - member);
+  PairItem cur = map_item(home, member);
+  PairItem nxt = map_item(home, 2 * L.members - 1 - member);
   bool draw = false;   // whether the item after the current one is drawn from the counter (every item but the first two)
   unsigned* const tickets = g_pair_tickets[L.slot];
   const uint64_t kstep = (uint64_t)kPBN * (uint64_t)p.k_ts * 2u, vstep = (uint64_t)kPBN * (uint64_t)p.v_ts * 2u;
@@ -481,6 +484,33 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   }
 
   unsigned tk = 0;   // thread 0: the ticket in flight
+  // The XCDs of a device do not run at one speed (their matrix throughput under this kernel differs by several percent), so
+  // a class served only by "its" workgroups finishes when its XCD does.  Lanes 0..7 of wave 0 therefore look at all the
+  // class counters once per item; when the home class is ahead of the class that has got least far by kStealLead tickets,
+  // the next draw is made from that class (its K/V then come through another XCD's L2: slower per tile, but work that
+  // the slowest XCD no longer has to do).  Towards the end of a class's list nothing is taken from it any more, so that
+  // every class ends on its own workgroups, by then at about the same time.
+  constexpr int kStealLead = 8;
+  unsigned snap = 0;      // wave 0, lane c: counter of class c as it was at the top of the current item
+  // t_tk[0]: the ticket; t_tk[1]: the class it was drawn from; t_tk[2]: the class the next draw is made from (kept in LDS:
+  // only wave 0 needs them, and the kernel has no registers to spare)
+  const bool balance = L.classes == 8 && (member & 15) == 0;
+  auto park_ticket = [&]() {   // wave 0, behind a barrier that has waited for the draw and the counter snapshot
+    if (tid == 0) t_tk[0] = (int)tk;
+    if (balance) {
+      int least = 0x7fffffff, who = home;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int v = (int)__builtin_amdgcn_readlane(snap, c);
+        if (v < least) {
+          least = v;
+          who = c;
+        }
+      }
+      const int own = (int)__builtin_amdgcn_readlane(snap, home);
+      if (tid == 0) t_tk[2] = (own >= least + kStealLead && least + 3 * L.members < n_items) ? who : home;
+    }
+  };
   // The barrier at the top of a tile, followed by a use of the ticket register: the barrier has waited for every memory
   // operation of the wave, the atomic included, and the (empty) use tells the compiler so; otherwise it would wait for the
   // atomic's result where the register is next written, at the top of the next item, and for everything issued before it.
@@ -502,7 +532,14 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     // The ticket of the item after next; thread 0 parks it in LDS behind the item's first barrier.  A wrapping increment
     // and not an addition: the compiler turns a uniform atomic addition into one lane's addition plus a broadcast of the
     // result, which would wait for the result right here.
-    if (tid == 0 && draw) tk = atomicInc(&tickets[cls], 0xffffffffu);
+    if (tid < 64 && draw) {
+      if (tid == 0) {
+        const int target = t_tk[2];
+        tk = atomicInc(&tickets[target], 0xffffffffu);
+        t_tk[1] = target;
+      }
+      if (balance && tid < 8) snap = __hip_atomic_load(&tickets[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -519,12 +556,12 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     const int my_tiles = wave_row0 + kPairWaveRows - 1 >= 0 ? min(ntiles, (wave_row0 + kPairWaveRows - 1) / kPBN + 1) : 0;
     const int unmasked = wave_row0 >= 0 ? (wave_row0 + 1) / kPBN : 0;
     uint64_t kbase = kv_base(cur, p.k, p.k_ts), vbase = kv_base(cur, p.v, p.v_ts);   // base of the tile after the one being computed
-    // The item's first barrier.  (Thread 0's wave has one more operation in flight, the draw; eight may stay in flight there
-    // too, which then makes it wait for one store.)  The ticket goes to LDS behind a barrier that has waited for the draw:
+    // The item's first barrier.  (Wave 0 has one or two more operations in flight, the draw and the look at the counters; eight
+    // may stay in flight there too, which then makes it wait for as many stores.)  The ticket goes to LDS behind a barrier that has waited for the draw:
     // the second one, or, for items of one or two tiles, here, where the compiler puts the wait in front of the write.
     if (stores8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else tile_barrier();
-    if (ntiles <= 2 && tid == 0 && draw) t_tk[0] = (int)tk;
+    if (ntiles <= 2 && tid < 64 && draw) park_ticket();
     int tile = 0;
     for (; tile < ntiles - 1; ++tile) {
       kbase += kstep;
@@ -541,7 +578,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
       else tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::false_type{}, my_row, nullptr);
       buf ^= 1;
       item_barrier();   // the top of the next tile
-      if (tile == 0 && ntiles > 2 && tid == 0 && draw) t_tk[0] = (int)tk;
+      if (tile == 0 && ntiles > 2 && tid < 64 && draw) park_ticket();
     }
     // the item's last tile: its successor is the next item's first tile, and the next item's Q operand comes with it.
     // Without a next item the loads are repeated on this item's own first tile and rows (harmless, never read).
@@ -550,7 +587,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
         // The ticket drawn at the top of the item went to LDS one barrier ago at the latest; an item of a single tile has
         // come through one barrier only and holds another one here.
         if (ntiles == 1) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        nxt = map_item(2 * L.members + __builtin_amdgcn_readfirstlane(t_tk[0]));
+        nxt = map_item(__builtin_amdgcn_readfirstlane(t_tk[1]), 2 * L.members + __builtin_amdgcn_readfirstlane(t_tk[0]));
       }
       const PairItem& to = nxt.valid ? nxt : cur;
       kbase = kv_base(to, p.k, p.k_ts);
