@@ -57,14 +57,14 @@ def test_prefill_other_scales_and_large_scores(gpu, ops, scale, qmul):
 def test_prefill_prescaled_q_form_meets_the_benchmark_tolerance(gpu):
     """MOPS_HIP_PREFILL_PRESCALE=1 (read once per process, hence the child process) selects the form that multiplies Q by
     scale * log2(e) once and rounds it back to bf16: faster, and within the benchmark's tolerance on the benchmark's
-    inputs, but its error grows with the size of the scores (at four times the benchmark's Q it leaves the tolerance)."""
+    inputs, but its error grows with the size of the scores (the figures at four times the benchmark's Q are printed)."""
     import os, subprocess, sys
     code = r'''
 import sys, torch
 sys.path.insert(0, ".")
 from nano_vllm_ninetoothed_amd import mops, workloads as W
 import oracle.mops_torch
-dev = torch.device("cuda:0")
+dev = torch.device("cuda:%d")
 hip = mops.get_op("flash_attn_varlen_func", "hip"); ref = mops.get_op("flash_attn_varlen_func", "torch")
 for qmul in (1.0, 4.0):
     d = W.prefill_inputs([333, 64, 700], seed=17)
@@ -75,7 +75,7 @@ for qmul in (1.0, 4.0):
     w = ref(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"], softmax_scale=d["scale"]).float()
     e = (o - w).abs()
     print(qmul, float(e.max()), float(e.mean()))
-'''
+''' % (gpu.index or 0)
     env = dict(os.environ, MOPS_HIP_PREFILL_PRESCALE="1")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=150)
@@ -84,7 +84,39 @@ for qmul in (1.0, 4.0):
     (q1, max1, mean1), (q4, max4, mean4) = [(float(a), float(b), float(c)) for a, b, c in rows]
     assert (q1, q4) == (1.0, 4.0)
     assert max1 <= 2e-2 and mean1 <= 2e-3, (max1, mean1)
-    assert mean4 > 2 * mean1, "the pre-scaled form is expected to lose accuracy as the scores grow"
+    print(f"pre-scaled Q form: mean-abs {mean1:.3g} at the benchmark's Q, {mean4:.3g} at four times it (max-abs {max4:.3g})")
+
+
+def test_prefill_row_form_still_matches_oracle(gpu):
+    """Plain causal prefill over grouped heads takes the two-heads-per-wave form (varlen_prefill_pair.hip); the 128-row form
+    stays the path of cached prefixes, odd group sizes and very large batches.  MOPS_HIP_PREFILL_FORM=rows (read once per
+    process, hence the child process) forces it for plain inputs too, so that its ragged and rectangular launches stay
+    covered against the oracle."""
+    import os, subprocess, sys
+    code = r'''
+import sys, torch
+sys.path.insert(0, ".")
+from nano_vllm_ninetoothed_amd import mops, workloads as W
+import oracle.mops_torch
+dev = torch.device("cuda:%d")
+hip = mops.get_op("flash_attn_varlen_func", "hip"); ref = mops.get_op("flash_attn_varlen_func", "torch")
+for lens in ([300, 1, 77, 513], [256, 256], [2048], [0, 31, 700, 64, 65, 1, 129] * 3):
+    d = W.prefill_inputs(lens, seed=sum(lens))
+    g = W.to_device(d, dev)
+    o = hip(g["q"], g["k"], g["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=g["cu_seqlens"], max_seqlen_k=d["max_seqlen"],
+            cu_seqlens_k=g["cu_seqlens"], softmax_scale=d["scale"], causal=True).cpu().float()
+    w = ref(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"], softmax_scale=d["scale"]).float()
+    e = (o - w).abs()
+    print(len(lens), float(e.max()), float(e.mean()))
+''' % (gpu.index or 0)
+    env = dict(os.environ, MOPS_HIP_PREFILL_FORM="rows")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=150)
+    assert out.returncode == 0, out.stderr[-2000:]
+    rows = [l.split() for l in out.stdout.strip().splitlines()[-4:]]
+    assert len(rows) == 4
+    for n, mx, mean in rows:
+        assert float(mx) <= 2e-2 and float(mean) <= 2e-3, (n, mx, mean)
 
 
 @pytest.mark.parametrize("nseq", [70, 200, 300])
@@ -99,6 +131,49 @@ def test_prefill_many_ragged_sequences(gpu, ops, nseq):
     lens[3] = 0
     d = W.prefill_inputs(lens, seed=nseq)
     assert_attention_close(_run(hip, d, gpu), _ref(ref, d), f"prefill {nseq} ragged sequences")
+
+
+def test_prefill_more_sequences_than_the_resident_form_holds(gpu, ops):
+    """Beyond 512 sequences the launch falls back to the 128-row form and its tile x sequence rectangle."""
+    hip, ref = ops("flash_attn_varlen_func")
+    gen = torch.Generator().manual_seed(600)
+    lens = torch.randint(0, 70, (600,), generator=gen).tolist()
+    lens[17] = 300
+    d = W.prefill_inputs(lens, hq=4, hkv=2, seed=600)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), "prefill 600 short sequences")
+
+
+def test_prefill_items_of_a_single_tile(gpu, ops):
+    """Sequences shorter than 64 tokens only: every work item of the resident form is a single K/V tile, so every draw of
+    the next item is waited for inside the item (the path with one more barrier), and every first tile is a partial one."""
+    hip, ref = ops("flash_attn_varlen_func")
+    gen = torch.Generator().manual_seed(5)
+    lens = torch.randint(1, 64, (400,), generator=gen).tolist()
+    d = W.prefill_inputs(lens, seed=5)
+    assert_attention_close(_run(hip, d, gpu), _ref(ref, d), "400 sequences of fewer than 64 tokens")
+
+
+def test_prefill_counter_rows_wrap_and_streams_overlap(gpu, ops):
+    """The resident form hands out work items through counters in device memory, one row of counters per launch, rows used
+    round robin (128 of them) and cleared by the last workgroup of a launch.  More launches than rows, then launches that
+    overlap on two streams: every result has the bits of the first launch."""
+    hip, _ = ops("flash_attn_varlen_func")
+    a = W.prefill_inputs([200, 64, 1, 333], seed=3)
+    b = W.prefill_inputs([129, 700], seed=4)
+    first_a, first_b = _run(hip, a, gpu).clone(), _run(hip, b, gpu).clone()
+    for i in range(300):
+        assert_bit_exact(_run(hip, a, gpu), first_a, f"launch {i}")
+    s1, s2 = torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)
+    torch.cuda.synchronize()
+    outs = []
+    for _ in range(20):
+        with torch.cuda.stream(s1):
+            outs.append((_run(hip, a, gpu), first_a))
+        with torch.cuda.stream(s2):
+            outs.append((_run(hip, b, gpu), first_b))
+    torch.cuda.synchronize()
+    for i, (got, want) in enumerate(outs):
+        assert_bit_exact(got, want, f"overlapping launch {i}")
 
 
 def test_prefill_ragged_batch_with_a_very_long_sequence(gpu, ops):
