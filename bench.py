@@ -12,8 +12,9 @@ A step is one flash_attn_with_kvcache call over the whole batch, KV cache reside
   copy = a plain 1 GiB device-to-device tensor copy (not a mops op): the known-size kernel against which
          the FETCH_SIZE / WRITE_SIZE counters of a profile are calibrated.
 
-The default line also carries an `e2e` block: the cfg5 workload's output tok/s with the decode step replayed from
-HIP graphs, once reading every step's tokens back (as the reference's loop does) and once pipelined (--no-e2e skips it).
+The default line also carries an `e2e` block: the cfg5 workload's output tok/s in three modes (eager with per-step
+readback, which is the reference's own setting; the decode step replayed from HIP graphs with per-step readback; the
+same pipelined) and the same engine on the torch-restated backend on a reduced run (--no-e2e skips the block).
 
 Prints ONE JSON line on stdout.  `roofline` is computed from HIP-event time of the op on its launch
 stream; `cpu_baseline` times the CPU restatement of the reference's torch backend (oracle/) on a
@@ -29,17 +30,31 @@ import time
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the default workload, calibrated against a 1 GiB copy
-DECODE_TRAFFIC_BYTES = 2497.6e6
-DECODE_TRAFFIC_SOURCE = "profiles/hbm_traffic_decode_prefill.txt (rocprofv3 --pmc, not measured by this run)"
-PREFILL_TRAFFIC_BYTES = {"prefill": 409.4e6, "prefill_long": 871.3e6}   # same source, same calibration
+TRAFFIC_PROFILE = "profiles/hbm_traffic_decode_prefill.txt"
+
+
+def profiled_traffic(section):
+    """HBM-side bytes per launch of a workload ("decode", "prefill", "prefill_long") as the committed rocprofv3 --pmc
+    summary states them (FETCH_SIZE + WRITE_SIZE, calibrated against a 1 GiB copy): the "total per launch" line of that
+    section.  Returns (bytes, source) or (None, reason): the figure is read, never re-typed, and it is a figure of that
+    profile, not of this run."""
+    import re
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, f"{TRAFFIC_PROFILE} not found"
+    m = re.search(r"^%s:\n(?:  .*\n)*?  total per launch: ([0-9.]+) MB" % re.escape(section), text, re.M)
+    if not m:
+        return None, f"no section '{section}' with a 'total per launch' line in {TRAFFIC_PROFILE}"
+    return float(m.group(1)) * 1e6, f"{TRAFFIC_PROFILE}, section '{section}' (rocprofv3 --pmc, not measured by this run)"
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 50; 500 for the prefill ops)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed warm-up steps (default 10; 300 for the prefill ops)")
     ap.add_argument("--op", default="decode",
                     choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "silu", "sampler", "qk_rope_store", "add_rms", "rms", "embedding", "copy", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
@@ -48,7 +63,17 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-e2e", action="store_true", help="default op only: skip the end-to-end block of the line (profiling runs)")
     ap.add_argument("--seed", type=int, default=0)
-    return ap.parse_args()
+    args = ap.parse_args()
+    # The prefill kernels keep the matrix pipes of all CUs busy, and the chip's power management answers the step from idle
+    # to that load with a transient: launches 10..150 of a back-to-back series run up to 40 % slower than the first ten
+    # and than everything after launch 250.  The warm-up of these ops is long enough to sit the transient out, and the
+    # timed series long enough not to be dominated by what is left of it.
+    matrix_bound = args.op in ("prefill", "prefill_long", "prefix_prefill")
+    if args.steps is None:
+        args.steps = 500 if matrix_bound else 50
+    if args.warmup is None:
+        args.warmup = 300 if matrix_bound else 10
+    return args
 
 
 def e2e_workload(n):
@@ -89,6 +114,27 @@ def e2e_modes(args, torch, modes):
     return {m: res[m] for m in modes}
 
 
+def e2e_comparison(args, torch, prompts, m=32, outlen=32):
+    """The same engine on the same GPU with the mops ops of the pure-torch restatement of the reference's torch backend,
+    next to the hip backend, on a reduced run (first m prompts, outlen output tokens each, no graphs).  It stands in for
+    the comparison the reference cannot offer: its triton backend has no decode attention (mops/triton/attention.py:150-168)."""
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    import oracle.mops_torch  # noqa: F401  comparison backend only
+    res = {}
+    for backend in ("hip", "torch"):
+        e = Engine(Qwen3Shape(), backend=backend, num_blocks=m * 6, seed=args.seed)
+        e.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 4)
+        _, s2 = e.generate(prompts[:m], outlen, temperature=0.6)
+        res[backend] = m * outlen / s2["total_s"]
+        del e
+        torch.cuda.empty_cache()
+    return {"what": "same engine, same GPU, no graphs, mops ops from the pure-torch restatement of the reference's torch backend "
+                    "(per-sequence attention loops) against the hip backend",
+            "sample": f"first {m} prompts, {outlen} output tokens each",
+            "hip_tok_per_s": round(res["hip"], 1), "torch_tok_per_s": round(res["torch"], 1),
+            "speedup": round(res["hip"] / res["torch"], 2)}
+
+
 E2E_WORKLOAD_TEXT = ("cfg5 end-to-end generate, random-init Qwen3-0.6B architecture (28 layers, hidden 1024, 16/8 heads, "
                      "vocab 151936, tied embeddings), mops hip backend, engine counterpart of the reference's bench.py:9-28")
 
@@ -112,20 +158,7 @@ def run_e2e(args, torch, dev, mops):
         "breakdown": r,
     }
     if not args.no_cpu_baseline:
-        import oracle.mops_torch  # noqa: F401  comparison backend only
-        m, outlen = 16, 16
-        res = {}
-        for backend in ("hip", "torch"):
-            e = Engine(Qwen3Shape(), backend=backend, num_blocks=m * 6, seed=args.seed)
-            e.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 4)
-            _, s2 = e.generate(prompts[:m], outlen, temperature=0.6)
-            res[backend] = m * outlen / s2["total_s"]
-            del e
-            torch.cuda.empty_cache()
-        out["comparison_baseline"] = {"what": "same engine, same GPU, mops ops from the pure-torch restatement of the reference's torch "
-                                              "backend (per-sequence attention loops)", "sample": f"first {m} prompts, {outlen} output tokens each",
-                                      "hip_tok_per_s": round(res["hip"], 1), "torch_tok_per_s": round(res["torch"], 1),
-                                      "speedup": round(res["hip"] / res["torch"], 2)}
+        out["comparison_baseline"] = e2e_comparison(args, torch, prompts)
     print(json.dumps(out))
 
 
@@ -211,8 +244,7 @@ def main():
         # launch shape, with its source next to it
         tuned = any(os.environ.get(v) for v in ("MOPS_HIP_DECODE_HPW", "MOPS_HIP_DECODE_NCOLS", "MOPS_HIP_DECODE_MIN_PER_COL"))
         if args.op == "decode" and args.seed == 0 and not tuned:
-            measured_traffic = DECODE_TRAFFIC_BYTES
-            traffic_source = DECODE_TRAFFIC_SOURCE
+            measured_traffic, traffic_source = profiled_traffic("decode")
 
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401
@@ -256,8 +288,7 @@ def main():
                   "total_tokens": sum(lens)}
         kernel_name = "varlen_prefill_kernel"
         if args.seed == 0:
-            measured_traffic = PREFILL_TRAFFIC_BYTES[args.op]
-            traffic_source = DECODE_TRAFFIC_SOURCE
+            measured_traffic, traffic_source = profiled_traffic(args.op)
 
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401
@@ -571,13 +602,17 @@ def main():
         out["roofline"]["library_gemm"] = {"what": "torch.matmul (hipBLASLt) bf16 8192^3, 20 launches back to back, same run",
                                            "TFLOP/s": round(gemm_tf, 1), "kernel_vs_library_gemm": round(achieved / gemm_tf, 4)}
     if args.op == "decode" and not args.no_e2e:
-        # second half of the headline metric: end-to-end output tok/s of the cfg5 workload, in the two graph modes
+        # second half of the headline metric: end-to-end output tok/s of the cfg5 workload.  "eager" is the reference's own
+        # setting (enforce_eager=True, bench.py:15 of the reference; every step's tokens read back,
+        # nanovllm/engine/model_runner.py:212); the two graph modes replay the decode step from HIP graphs.
         step = op = caches = q = None
         torch.cuda.empty_cache()
-        r = e2e_modes(args, torch, ["stepwise", "pipelined"])
+        r = e2e_modes(args, torch, ["eager", "stepwise", "pipelined"])
         out["e2e"] = {"metric": "e2e_output_tok_per_s", "unit": "tok/s", "workload": E2E_WORKLOAD_TEXT,
                       "prompts": args.e2e_seqs, "prompt_len": "uniform[100,1024]", "max_tokens": "uniform[100,1024]",
-                      "temperature": 0.6, "runs": [r["stepwise"], r["pipelined"]]}
+                      "temperature": 0.6, "runs": [r["eager"], r["stepwise"], r["pipelined"]]}
+        if not args.no_cpu_baseline:
+            out["e2e"]["comparison_baseline"] = e2e_comparison(args, torch, e2e_workload(args.e2e_seqs)[0])
     print(json.dumps(out))
 
 

@@ -32,16 +32,33 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(
   const uint16_t* xp = qkv + t * qkv_token_stride + (int64_t)hd * kFusedDim + (lane << 3);
   u32x4 a = {0u, 0u, 0u, 0u};
   if (row_ok) a = load16_stream(xp);
+  // Everything else the row needs is requested here as well, in front of the reduction and not behind it: the norm
+  // weight, the token's cos / sin, its cache slot.  At decode sizes the kernel lives a few microseconds, and each
+  // further trip to memory behind the statistics was a third of that.
+  const bool is_q = hd < hq;
+  const bool is_v = hd >= hq + hkv;
+  int slot = -1;
+  if (row_ok && !is_q) slot = slot_mapping[t];
+  u32x4 w = {0u, 0u, 0u, 0u};
+  f32x4 cv[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, sv[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  if (!is_v) {
+    w = load16((is_q ? q_weight : k_weight) + (lane << 3));
+    const float* cp = cos + t * cos_token_stride + ((lane & 7) << 3);
+    const float* sp = sin + t * sin_token_stride + ((lane & 7) << 3);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      cv[h] = *reinterpret_cast<const f32x4*>(cp + 4 * h);
+      sv[h] = *reinterpret_cast<const f32x4*>(sp + 4 * h);
+    }
+  }
 
-  if (hd >= hq + hkv) {   // a v head: straight into the cache
+  if (is_v) {   // a v head: straight into the cache
     if (row_ok) {
-      const int slot = slot_mapping[t];
       if (slot >= 0 && slot < num_slots)
         store16(v_cache + ((int64_t)slot * hkv + (hd - hq - hkv)) * kFusedDim + (lane << 3), a);
     }
     return;   // rows of one head type fill whole 16-lane groups, so the shuffles below never miss a lane
   }
-  const bool is_q = hd < hq;
 
   // ---- RMSNorm, as rmsnorm_kernel<16, 1, false>
   float v[8];
@@ -56,7 +73,6 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(
   }
   ss = group_sum<16>(ss);
   const float rstd = 1.0f / sqrtf(ss / (float)kFusedDim + eps);
-  const u32x4 w = load16((is_q ? q_weight : k_weight) + (lane << 3));
   u32x4 nrm;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
@@ -70,14 +86,12 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(
 #pragma unroll
   for (int e = 0; e < 4; ++e) other[e] = (unsigned)__shfl_xor((int)nrm[e], 8, kWave);
   const bool upper = lane >= 8;
-  const float* cp = cos + t * cos_token_stride + ((lane & 7) << 3);
-  const float* sp = sin + t * sin_token_stride + ((lane & 7) << 3);
   u32x4 o;
   {
 #pragma clang fp contract(off)  // products and sums stay separate roundings, as in the library expression
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float c0 = cp[2 * e], c1 = cp[2 * e + 1], s0 = sp[2 * e], s1 = sp[2 * e + 1];
+      const float c0 = cv[e >> 1][2 * (e & 1)], c1 = cv[e >> 1][2 * (e & 1) + 1], s0 = sv[e >> 1][2 * (e & 1)], s1 = sv[e >> 1][2 * (e & 1) + 1];
       const float ml = bf16lo_to_f32(nrm[e]), mh = bf16hi_to_f32(nrm[e]);       // this lane's half
       const float ol = bf16lo_to_f32(other[e]), oh = bf16hi_to_f32(other[e]);   // the partner's half
       float yl, yh;
@@ -97,7 +111,6 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(
   } else {
     const int kh = hd - hq;
     if (k_out) store16(k_out + (t * hkv + kh) * (int64_t)kFusedDim + (lane << 3), o);
-    const int slot = slot_mapping[t];
     if (slot >= 0 && slot < num_slots) store16(k_cache + ((int64_t)slot * hkv + kh) * kFusedDim + (lane << 3), o);
   }
 }
@@ -120,8 +133,8 @@ extern "C" int mops_hip_qk_norm_rope_store(const void* qkv, int64_t qkv_token_st
     return MOPS_HIP_EINVAL;
   if (qkv_token_stride & 7) return MOPS_HIP_EALIGN;
   if (!aligned16(qkv) || !aligned16(q_weight) || !aligned16(k_weight) || !aligned16(q_out) || (k_out && !aligned16(k_out)) ||
-      !aligned16(k_cache) || !aligned16(v_cache) || (reinterpret_cast<uintptr_t>(cos) & 3u) || (reinterpret_cast<uintptr_t>(sin) & 3u))
-    return MOPS_HIP_EALIGN;
+      !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(cos) || !aligned16(sin) || (cos_token_stride & 3) || (sin_token_stride & 3))
+    return MOPS_HIP_EALIGN;   // cos / sin are read as 16-byte pieces
   if (heads > 4096 || tokens > (int64_t)1 << 40 || num_slots * hkv > ((int64_t)1 << 40)) return MOPS_HIP_EUNSUPPORTED;
   const int64_t rows = tokens * heads;
   const int64_t grid = (rows + kFusedThreads / 16 - 1) / (kFusedThreads / 16);

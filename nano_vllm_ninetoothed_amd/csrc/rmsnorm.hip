@@ -33,15 +33,19 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
   const uint16_t* rr = FUSE_ADD ? residual + (row_ok ? row : 0) * r_row_stride : nullptr;
 
   float v[ITERS][8];
+  u32x4 wv[ITERS];   // the weight pieces are requested together with the row, not behind the reduction: at decode
+                     // sizes the kernel's whole life is a few microseconds and a second trip to memory is a third of it
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int p = lane + it * GROUP;
     const bool ok = row_ok && p < pieces;
     u32x4 a = {0u, 0u, 0u, 0u}, b = {0u, 0u, 0u, 0u};
+    wv[it] = u32x4{0u, 0u, 0u, 0u};
     if (ok) {
       a = load16_stream(xr + (p << 3));
       if (FUSE_ADD) b = load16_stream(rr + (p << 3));
+      wv[it] = load16(weight + (p << 3));
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -80,7 +84,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(
   for (int it = 0; it < ITERS; ++it) {
     const int p = lane + it * GROUP;
     if (row_ok && p < pieces) {
-      const u32x4 w = load16(weight + (p << 3));
+      const u32x4 w = wv[it];
       u32x4 o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {

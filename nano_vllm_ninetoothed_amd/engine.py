@@ -75,9 +75,9 @@ class Sequence:
 
 
 class Engine:
-    def __init__(self, shape: Qwen3Shape = Qwen3Shape(), backend: str = "hip", num_blocks: int = 2560, seed: int = 0,
+    def __init__(self, shape: Qwen3Shape | None = None, backend: str = "hip", num_blocks: int = 2560, seed: int = 0,
                  max_num_batched_tokens: int = 16384, max_num_seqs: int = 512, device="cuda:0"):
-        self.shape = s = shape
+        self.shape = s = shape if shape is not None else Qwen3Shape()
         self.dev = torch.device(device)
         self.backend = backend
         self.max_num_batched_tokens = max_num_batched_tokens
@@ -130,6 +130,24 @@ class Engine:
         self.last_tok = torch.zeros(max_num_seqs + 1, dtype=torch.int64, device=self.dev)
         self.free_rows = deque(range(1, max_num_seqs + 1))
         self.unit_temps = torch.ones(max_num_seqs, dtype=torch.float32, device=self.dev)
+        self._sampler_checked = False
+        self.capture_stream = None
+
+    def _check_sampler_ignores_temperature(self):
+        """Pipelined generation hands the sampler unit temperatures (the per-sequence ones would cost a gather per step).
+        That is only right while the backend's sampler is greedy, as the reference's is (mops/torch/ops.py:37-43 with
+        the sampling line commented out): checked once, on random logits, before the first pipelined run."""
+        if self._sampler_checked:
+            return
+        g = torch.Generator(device=self.dev).manual_seed(1234)
+        logits = torch.randn((8, 4096), generator=g, device=self.dev, dtype=torch.float32).to(torch.bfloat16)
+        hot = torch.full((8,), 0.3, dtype=torch.float32, device=self.dev)
+        a = self.op_sampler_forward(logits, self.unit_temps[:8])
+        b = self.op_sampler_forward(logits, hot)
+        if not torch.equal(a, b):
+            raise RuntimeError(f"the {self.backend} backend's sampler depends on the temperature: pipelined generation "
+                               "passes unit temperatures and would sample differently; set engine.pipelined = False")
+        self._sampler_checked = True
 
     # ------------------------------------------------------------------ HIP graphs for decode
     @torch.inference_mode()
@@ -159,7 +177,9 @@ class Engine:
         # Every bucket is captured on one stream of our own.  The ops keep their scratch buffers per stream, and
         # the graphs hold those addresses: sizing the scratch for the largest bucket on that stream before the
         # first capture means no capture, in whatever order, allocates or moves it.
-        capture_stream = torch.cuda.Stream(dev)
+        # The stream stays alive with the engine: the scratch is keyed by the stream's handle, and a handle that went back
+        # to torch's pool could be handed to unrelated eager work, which would then share the graphs' scratch.
+        capture_stream = self.capture_stream = self.capture_stream or torch.cuda.Stream(dev)
         if self.backend == "hip":
             from .mops.hip.ops import reserve_decode_workspace
             with torch.cuda.stream(capture_stream):
@@ -327,6 +347,7 @@ class Engine:
     def _generate_pipelined(self, stats):
         """Runs until no sequence is waiting or running without reading a token back in between."""
         import numpy as np
+        self._check_sampler_ignores_temperature()
         dev = self.dev
         n, max_blocks = self.g_ids.numel(), self.g_tables.size(1)
         depth = 8                                  # steps the host may be ahead of the GPU

@@ -31,6 +31,25 @@ def test_store_kvcache_matches_oracle(gpu, ops, n_tokens, v_stride):
     assert_bit_exact(vc_g, vc, "v_cache")
 
 
+def test_store_kvcache_benchmark_token_count(gpu, ops):
+    """The store of the prefill benchmark exactly as it is drawn: T = the sum of the 16 seeded sequence lengths
+    (uniform in [128, 2048], seed 0) = 20514 tokens, V a view with row stride 4096, random-permutation slots; bit-exact
+    against the scatter of mops/triton/attention.py:30-38."""
+    hip, ref = ops("store_kvcache")
+    T = sum(W.random_seq_lens(16, 128, 2048, seed=0))
+    assert T == 20514
+    d = W.store_inputs(T, seed=0, v_row_stride=4096)
+    kc, vc = _caches(d["num_blocks"], d["hkv"])
+    ref(d["key"], d["value"], kc, vc, d["slot_mapping"])
+    kc_g, vc_g = (t.to(gpu) for t in _caches(d["num_blocks"], d["hkv"]))
+    wide = d["value"]._base.to(gpu)
+    value_g = wide[:, 4096 - d["hkv"] * W.HEAD_DIM:].view(T, d["hkv"], W.HEAD_DIM)
+    assert value_g.stride(0) == 4096
+    hip(d["key"].to(gpu), value_g, kc_g, vc_g, d["slot_mapping"].to(gpu))
+    assert_bit_exact(kc_g, kc, "k_cache")
+    assert_bit_exact(vc_g, vc, "v_cache")
+
+
 def test_store_kvcache_skips_minus_one_and_keeps_other_slots(gpu, ops):
     hip, ref = ops("store_kvcache")
     d = W.store_inputs(300, seed=5)

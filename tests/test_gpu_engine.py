@@ -177,3 +177,27 @@ def test_full_size_engine_pipelined_equals_stepwise(gpu):
         assert stats["decode_tokens"] + 64 == sum(max_tokens)       # the first token of a sequence comes from its prefill
         runs.append(outs)
     assert runs[0] == runs[1], "pipelined and stepwise generation disagree"
+
+
+def test_end_to_end_workload_exactly_as_the_reference_words_it(gpu):
+    """The end-to-end configuration at its full size (bench.py:9-28 of the reference): random.seed(0), 256 prompts of
+    100..1024 random token ids, 100..1024 output tokens each, temperature 0.6, no EOS, on the random-init Qwen3-0.6B
+    architecture.  One engine runs it pipelined and then stepwise: the tokens must be equal, every sequence gets exactly
+    its max_tokens, every cache block comes back."""
+    import random
+    from nano_vllm_ninetoothed_amd.engine import Engine, Qwen3Shape
+    random.seed(0)
+    prompts = [[random.randint(0, 10000) for _ in range(random.randint(100, 1024))] for _ in range(256)]
+    max_tokens = [random.randint(100, 1024) for _ in range(256)]
+    eng = Engine(Qwen3Shape(), backend="hip", num_blocks=2560, seed=0, device=str(gpu))
+    eng.generate([[1, 2, 3, 4, 5, 6, 7, 8]], 8)
+    eng.capture_decode_graphs(max_bs=256, max_model_len=4096)
+    runs = []
+    for pipelined in (True, False):
+        eng.pipelined = pipelined
+        outs, stats = eng.generate(prompts, max_tokens, temperature=0.6)
+        assert [len(o) for o in outs] == max_tokens
+        assert len(eng.free_blocks) == eng.num_blocks and not eng.running and not eng.waiting
+        assert stats["decode_tokens"] + 256 == sum(max_tokens)
+        runs.append(outs)
+    assert runs[0] == runs[1], "pipelined and stepwise generation disagree on the full workload"
