@@ -11,6 +11,7 @@ A step is one flash_attn_with_kvcache call over the whole batch, KV cache reside
          temperature 0.6, no EOS): output tokens per second; --steps/--warmup are ignored.
   copy = a plain 1 GiB device-to-device tensor copy (not a mops op): the known-size kernel against which
          the FETCH_SIZE / WRITE_SIZE counters of a profile are calibrated.
+  launch_floor = an empty kernel: the floor under the durations of the small operators (value 0, read the time).
 
 The default line also carries an `e2e` block: the cfg5 workload's output tok/s in three modes (eager with per-step
 readback, which is the reference's own setting; the decode step replayed from HIP graphs with per-step readback; the
@@ -56,7 +57,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 50; 500 for the prefill ops)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed warm-up steps (default 10; 300 for the prefill ops)")
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "silu", "sampler", "qk_rope_store", "add_rms", "rms", "embedding", "copy", "e2e"])
+                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "silu", "sampler", "qk_rope_store", "add_rms", "rms", "embedding", "copy", "launch_floor", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
@@ -493,6 +494,19 @@ def main():
             t0 = time.perf_counter()
             ref(st["qkv"], qw.cpu(), kw.cpu(), 1e-6, cos.cpu(), sin.cpu(), st["kc"], st["vc"], st["slots"], hq, hkv, need_k=False)
             return time.perf_counter() - t0, "whole batch, one run", work
+
+    elif args.op == "launch_floor":
+        # an empty kernel: the floor under the durations of the small operators
+        lib = _capi.load()
+
+        def step(i):
+            return lib.mops_hip_launch_floor(torch.cuda.current_stream(dev).cuda_stream)
+
+        work = 0.0
+        metric, unit = "launch_floor_GBps", "GB/s"
+        config = {"workload": "an empty kernel (64 lanes), launches back to back: what a launch costs with nothing to do"}
+        kernel_name = "launch_floor_kernel"
+        cpu_fn = None
 
     elif args.op == "copy":
         nbytes = 1 << 30

@@ -254,6 +254,13 @@ int mops_hip_sampler_argmax(const void* logits, int64_t row_stride, int64_t* out
                             void* stream);
 
 /*
+ * An empty kernel on `stream`: what one launch costs on this device with nothing to do.  No counterpart in the
+ * reference; it exists so that the durations of the small operators (norms, embedding at decode sizes) can be read
+ * against a measured floor (bench.py --op launch_floor).
+ */
+int mops_hip_launch_floor(void* stream);
+
+/*
  * qk_norm_rope_store — the four small steps between the qkv projection and the attention call of a Qwen3
  * layer as one launch: per-head RMSNorm of q and k, rotary embedding of both, scatter of k and v into the
  * paged cache.  Replaces the sequence nanovllm/models/qwen3.py:74-80 (q_norm, k_norm, rotary_emb) +

@@ -46,6 +46,7 @@ SIGNATURES = {
     "mops_hip_apply_rotary_emb": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p]),
     "mops_hip_sampler_argmax": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
+    "mops_hip_launch_floor": (c_int, [c_void_p]),
     "mops_hip_qk_norm_rope_store": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                             c_int64, c_int64, c_float, c_void_p]),
@@ -55,7 +56,7 @@ SIGNATURES = {
     "mops_hip_linear_tune": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
 }
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lib = None
 

@@ -17,7 +17,7 @@ int record_hip_error(hipError_t e) {
 }
 }  // namespace mops
 
-extern "C" int mops_hip_abi_version(void) { return 8; }
+extern "C" int mops_hip_abi_version(void) { return 9; }
 
 extern "C" int mops_hip_last_hip_error(void) { return mops::g_last_hip_error; }
 

@@ -212,3 +212,14 @@ extern "C" int mops_hip_sampler_argmax(const void* logits, int64_t row_stride, i
                      (const uint16_t*)logits, row_stride, out, (int)n);
   return finish_launch();
 }
+
+// An empty kernel: what a launch costs on this device with nothing to do, as a floor to read the small operators'
+// durations against (bench.py --op launch_floor).
+namespace mops {
+__global__ void launch_floor_kernel() {}
+}  // namespace mops
+
+extern "C" int mops_hip_launch_floor(void* stream) {
+  hipLaunchKernelGGL(mops::launch_floor_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream);
+  return mops::finish_launch();
+}
