@@ -608,7 +608,9 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
         tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::true_type{}, my_row, qnext);
       }
     }
-    item_barrier();   // every wave is done with the last tile: its buffer pair is free for the epilogue
+    // Every wave is done with the last tile: its buffer pair is free for the epilogue.  Only LDS traffic is waited for:
+    // the loads in flight are the next item's (into the other buffer pair and into qb), which the epilogue does not touch.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
     // ---- epilogue.  A lane holds 8-byte pieces of its own column, which would make every store instruction touch 64
     //      cache lines; the wave's 32 columns x 256 bytes go through LDS instead (the wave's quarter of the last tile's
