@@ -29,6 +29,7 @@ constexpr int kPairRows = 64;          // q rows per item
 constexpr int kPairWaveRows = 16;      // q rows per wave (x 2 heads = 32 MFMA columns)
 constexpr int kPairMaxBatch = 512;     // sequences per launch (their offsets live in LDS)
 constexpr int kPairMaxTiles = 1024;    // q tiles per sequence (65536 tokens)
+constexpr int kPairTable = 1024;       // (q tile, sequence) pairs whose rank -> pair mapping is tabulated in LDS
 constexpr int kPairSlots = 128;        // launches that may overlap on one device (one counter row each)
 
 // Item counters, one row per slot: [c] next ticket of class c (the workgroups with id % classes == c), [8] workgroups
@@ -39,6 +40,7 @@ struct PairLaunch {
   int classes;          // 8 when there are 8 kv heads (class = kv head = XCD), else 1
   int units_per_class;  // head pairs per class
   int units_per_kv;     // head pairs per kv head (group / 2)
+  int upc_shift;        // log2(units_per_class) when that is a power of two, else -1
   int members;          // workgroups per class
   int q_tiles;          // bound on the q tiles (64 rows) of a sequence
   int slot;             // counter row
@@ -54,7 +56,7 @@ __device__ __forceinline__ void q_piece_async(bf16x8& dst, const char* ptr) {
 }
 
 struct PairItem {
-  int valid, seq_begin, seq_len, q0, unit;
+  int valid, seq_begin, seq_len, q0, unit, kv;   // unit: the head pair 2u, 2u + 1; kv: its kv head
 };
 
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const PrefillParams p, const PairLaunch L) {
@@ -63,12 +65,14 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   const float ec = fmaxf(fabsf(p.scale_log2), 1e-30f);
   // One array, so that the tile buffers start at the workgroup's LDS offset 0: a direct-to-LDS load takes its destination
   // from M0 as a plain offset.  K[2] then V[2] (16 KiB each), then the tables of the rank -> item mapping.
-  constexpr int kTabCu = 0, kTabCnt = kPairMaxBatch + 4, kTabFrom = kTabCnt + kPairMaxBatch, kTabTicket = kTabFrom + kPairMaxTiles + 4;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPTile + (kTabTicket + 4) * 4];
+  constexpr int kTabCu = 0, kTabCnt = kPairMaxBatch + 4, kTabFrom = kTabCnt + kPairMaxBatch, kTabTicket = kTabFrom + kPairMaxTiles + 4,
+                kTabPair = kTabTicket + 4;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPTile + (kTabPair + kPairTable) * 4];
   int* const tab = reinterpret_cast<int*>(lds + 4 * kPTile);
   int* const t_cu = tab + kTabCu;        // cu_seqlens [batch + 1]
   int* const t_cnt = tab + kTabCnt;      // q tiles of sequence b
   int* const t_from = tab + kTabFrom;    // (q tile, sequence) pairs whose q tile index is >= l, l = 0 .. q_tiles + 1
+  int* const t_pair = tab + kTabPair;    // pair of rank r as (sequence << 16 | q tile), when the launch is small enough for the table
   int* const t_tk = tab + kTabTicket;    // the ticket drawn during the current item
   unsigned char* const lds_k = lds;
   unsigned char* const lds_v = lds + 2 * kPKTile;
@@ -90,41 +94,55 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     t_cnt[b] = (qs >= 0 && len > 0) ? min((len + kPairRows - 1) / kPairRows, L.q_tiles) : 0;
   }
   __syncthreads();
+  // Small launches also tabulate rank -> pair, a lookup per item instead of two searches: the thread that works out
+  // from[l] knows where the pairs of q tile l - 1 start (at rank from[l]) and writes them down, sequences in order.
+  const bool tabulated = p.batch <= 64 && (p.total_tokens >> 6) + p.batch <= kPairTable;
   for (int l = tid; l <= L.q_tiles + 1; l += kPThreads) {
     int s = 0;
     if (l < L.q_tiles)
       for (int b = 0; b < p.batch; ++b) s += max(0, t_cnt[b] - l);
     t_from[l] = s;
+    if (tabulated && l >= 1 && l <= L.q_tiles) {
+      for (int b = 0; b < p.batch; ++b)
+        if (t_cnt[b] > l - 1) t_pair[s++] = (b << 16) | (l - 1);
+    }
   }
   __syncthreads();
   const int home = (int)blockIdx.x % L.classes;   // the class this workgroup serves first
   const int member = (int)blockIdx.x / L.classes;
-  const int n_items = __builtin_amdgcn_readfirstlane(t_from[0]) * L.units_per_class;   // items of a class (the same for all)
+  const int n_pairs = __builtin_amdgcn_readfirstlane(t_from[0]);
+  const int n_items = n_pairs * L.units_per_class;   // items of a class (the same for all)
   if (tid == 0) t_tk[2] = home;
 
   // rank (within the class, heaviest first) -> item.  Every wave works it out for itself; all values are wave-uniform.
   auto map_item = [&](int cls, int R) -> PairItem {
-    PairItem it = {0, 0, 0, 0, 0};
+    PairItem it = {0, 0, 0, 0, 0, 0};
     if (R >= n_items) return it;
-    const int pr = R / L.units_per_class;                       // rank of the (q tile, sequence) pair
-    const int unit = cls * L.units_per_class + R % L.units_per_class;
+    // rank of the (q tile, sequence) pair and the head pair inside the class (no division for 1, 2, 4 .. pairs per class)
+    const int pr = L.upc_shift >= 0 ? R >> L.upc_shift : R / L.units_per_class;
+    const int unit = cls * L.units_per_class + (R - pr * L.units_per_class);
+    int m, b = -1;
+    if (tabulated) {
+      const int e = t_pair[pr];
+      m = e & 0xffff;
+      b = e >> 16;
+    } else {
     // the pair's q tile index m: the largest l with from[l] > pr; from[] is non-increasing, two levels of 64-way search
     const int S = (L.q_tiles + 64) >> 6;
-    const int i1 = lane * S;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));   // opaque: keeps the compiler from holding the LDS addresses of the searches in registers for the whole kernel
+    const int i1 = ln * S;
     const int v1 = i1 <= L.q_tiles ? t_from[i1] : 0;
     const unsigned long long m1 = __ballot(v1 > pr);
     if (m1 == 0) return it;
-    int m = (63 - __builtin_clzll(m1)) * S;
+    m = (63 - __builtin_clzll(m1)) * S;
     if (S > 1) {
-      const int i2 = m + lane;
-      const int v2 = (lane < S && i2 <= L.q_tiles) ? t_from[i2] : 0;
+      const int i2 = m + ln;
+      const int v2 = (ln < S && i2 <= L.q_tiles) ? t_from[i2] : 0;
       const unsigned long long m2 = __ballot(v2 > pr);
       m += 63 - __builtin_clzll(m2 | 1ull);
     }
     int r = pr - t_from[m + 1];   // rank among the sequences that have q tile m
-    int b = -1;
-    int ln = lane;
-    asm volatile("" : "+v"(ln));   // opaque: keeps the compiler from holding this loop's LDS addresses in registers for the whole kernel
     for (int j = 0; 64 * j < p.batch && b < 0; ++j) {
       const int bb = ln + 64 * j;
       const bool has = bb < p.batch && t_cnt[bb] > m;
@@ -138,6 +156,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
         r -= c;
       }
     }
+    }
     if (b < 0) return it;
     const int seq_begin = t_cu[b];
     const int seq_len = min(t_cu[b + 1], p.total_tokens) - seq_begin;
@@ -149,6 +168,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     it.seq_len = __builtin_amdgcn_readfirstlane(seq_len);
     it.q0 = __builtin_amdgcn_readfirstlane(seq_len - (seq_tiles - m) * kPairRows);
     it.unit = __builtin_amdgcn_readfirstlane(unit);
+    it.kv = L.classes == 8 ? cls : it.unit / L.units_per_kv;
     return it;
   };
 
@@ -234,8 +254,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     }
   };
   auto kv_base = [&](const PairItem& it, const uint16_t* base, int64_t ts) -> uint64_t {
-    const int g = it.unit / L.units_per_kv;
-    return reinterpret_cast<uint64_t>(base) + (uint64_t)(((int64_t)it.seq_begin * ts + (int64_t)g * kPD) * 2);
+    return reinterpret_cast<uint64_t>(base) + (uint64_t)(((int64_t)it.seq_begin * ts + (int64_t)it.kv * kPD) * 2);
   };
 
   // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
@@ -680,6 +699,9 @@ int launch_prefill_pair(const PrefillParams& p, hipStream_t stream) {
   L.classes = p.hkv == 8 ? 8 : 1;
   L.units_per_class = units / L.classes;
   L.units_per_kv = p.group / 2;
+  L.upc_shift = -1;
+  for (int sft = 0; sft < 16; ++sft)
+    if (L.units_per_class == (1 << sft)) L.upc_shift = sft;
   static std::atomic<int> cu_count[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MOPS_HIP_EUNSUPPORTED;
