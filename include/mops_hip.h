@@ -144,8 +144,12 @@ int mops_hip_attn_paged_decode_bf16(const void* q, int64_t q_batch_stride,
  * cut over the workgroups) depends only on cache_seqlens, the batch and head counts and the block size, not
  * on q or on the caches, so the layers of one decode step can share it: call the first layer with
  * MOPS_HIP_DECODE_PLAN_AND_ATTEND and the others, on the same stream with the same workspace and the same
- * metadata, with MOPS_HIP_DECODE_REUSE_PLAN.  No counterpart in the reference (its attention call is per layer,
- * nanovllm/layers/attention.py:40-42).
+ * metadata, with MOPS_HIP_DECODE_REUSE_PLAN.  "The same metadata" means the same CONTENTS: a plan records the batch and
+ * the head geometry it was made for (a call whose batch or heads differ is refused: its output is zeros), but not the
+ * lengths.  If cache_seqlens or block_table have been rewritten in place since the planning call (same pointers, new
+ * values, as a serving loop's static buffers are), MOPS_HIP_DECODE_REUSE_PLAN follows the old split: rows come out
+ * truncated or zero, and nothing reports it.  Plan again whenever the contents may have changed (once per decode
+ * step).  No counterpart in the reference (its attention call is per layer, nanovllm/layers/attention.py:40-42).
  */
 #define MOPS_HIP_DECODE_PLAN_AND_ATTEND 0
 #define MOPS_HIP_DECODE_REUSE_PLAN 1

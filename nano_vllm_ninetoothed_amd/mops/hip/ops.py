@@ -195,7 +195,11 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     reuse_plan (extension): skip the planning kernel and use the split the last planning call on this stream left
     in the scratch.  Only valid when that call had the same cache_seqlens and block_table tensors and the same
     head geometry, i.e. for layers 2..N of one decode step; anything else raises ValueError.  (The kernels
-    themselves refuse a plan whose recorded batch or head geometry differs from their launch and write zeros.)"""
+    themselves refuse a plan whose recorded batch or head geometry differs from their launch and write zeros.)
+    The check compares tensors by address and shape, not by value: cache_seqlens and block_table must also still
+    HOLD what the planning call saw.  A caller that rewrites them in place (static graph buffers) and then passes
+    reuse_plan=True without planning again gets the old split applied to the new lengths - truncated or zero rows,
+    silently.  Plan once per decode step, as the engine counterpart does at layer 0."""
     _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
     _require(cache_seqlens is not None and block_table is not None, "cache_seqlens and block_table are required")
     _require_cuda_bf16("q", q)

@@ -295,6 +295,31 @@ def test_reuse_plan_without_a_matching_plan_is_refused(gpu, ops):
     hip(d1["q"], d1["k_cache"], d1["v_cache"], reuse_plan=True, **kw1)            # the matching one is accepted
 
 
+def test_lengths_rewritten_in_place_need_a_new_plan(gpu, ops):
+    """The static-buffer pattern of a serving loop: cache_seqlens and block_table keep their addresses and are rewritten
+    in place between decode steps.  The reuse_plan check compares addresses, so it cannot see that; the contract is that
+    the first layer of every step plans again.  Doing so gives the oracle's answer for the new lengths, and the layers
+    that then reuse the plan give the bits of calls that plan for themselves.  (Reusing the OLD plan after the rewrite is
+    the caller's error: it would cut the new lengths by the old split; it is documented, not detected.)"""
+    hip, ref = ops("flash_attn_with_kvcache")
+    ctx_a, ctx_b = [900, 2100, 64, 3000, 1], [901, 2101, 65, 3001, 2]        # the next step: every sequence one longer
+    da, db = W.decode_inputs(ctx_a, seed=41), W.decode_inputs(ctx_b, seed=41)
+    g = W.to_device(da, gpu)
+    kw = dict(cache_seqlens=g["cache_seqlens"], block_table=g["block_table"], softmax_scale=da["scale"], causal=True)
+    hip(g["q"], g["k_cache"], g["v_cache"], **kw)                                     # step t, layer 0: plans
+    hip(g["q"], g["k_cache"], g["v_cache"], reuse_plan=True, **kw)                    # step t, layer 1
+    gb = W.to_device(db, gpu)
+    assert gb["block_table"].shape == g["block_table"].shape
+    g["cache_seqlens"].copy_(gb["cache_seqlens"])                                     # in place: same addresses
+    g["block_table"].copy_(gb["block_table"])
+    got0 = hip(gb["q"], gb["k_cache"], gb["v_cache"], **kw)                           # step t+1, layer 0: plans again
+    got1 = hip(gb["q"], gb["k_cache"], gb["v_cache"], reuse_plan=True, **kw)          # step t+1, layer 1: reuses
+    want = ref(db["q"], db["k_cache"], db["v_cache"], cache_seqlens=db["cache_seqlens"], block_table=db["block_table"],
+               softmax_scale=db["scale"], causal=True)
+    assert_attention_close(got0, want, "decode after an in-place rewrite of the lengths, planned again")
+    assert_bit_exact(got1, got0, "the next layer on the renewed plan")
+
+
 def test_kernels_refuse_a_plan_made_for_another_launch(gpu):
     """Through the C ABI, where nothing tracks the plan: MOPS_HIP_DECODE_REUSE_PLAN on a workspace that was never
     planned, or was planned for a larger batch, must not follow the stale sequence indices.  The kernels compare the

@@ -59,6 +59,40 @@ def test_no_alloc_decode_matches_workspace_decode_twice(gpu, ops):
         assert_attention_close(got, oracle, f"no-alloc decode vs oracle, {len(ctx)} sequences")
 
 
+def test_no_alloc_decode_allocates_nothing_and_can_be_captured(gpu):
+    """What the entry point exists for: a call after the first one on a device takes no device memory (neither from the
+    driver nor from torch's allocator), and it can be recorded into a HIP graph (the first call, which looks up the
+    scratch's address, has happened before); every replay gives the eager call's bits."""
+    lib = _capi.load()
+    d = W.decode_inputs([700, 1, 33, 2049, 256, 4000], seed=23)
+    g = W.to_device(d, gpu)
+    out = torch.full_like(g["q"], float("nan"))
+    args = _args(g, out)
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+    _capi.check("warm-up", lib.mops_hip_attn_paged_decode_noalloc_bf16(*args, d["scale"], stream))
+    torch.cuda.synchronize()
+    eager = out.clone()
+    free0, _ = torch.cuda.mem_get_info(gpu)
+    alloc0, reserved0 = torch.cuda.memory_allocated(gpu), torch.cuda.memory_reserved(gpu)
+    for _ in range(3):
+        _capi.check("call", lib.mops_hip_attn_paged_decode_noalloc_bf16(*args, d["scale"], stream))
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info(gpu)
+    assert (torch.cuda.memory_allocated(gpu), torch.cuda.memory_reserved(gpu)) == (alloc0, reserved0)
+    assert free1 == free0, f"device memory in use changed by {free0 - free1} bytes across allocation-free calls"
+    assert_bit_exact(out, eager, "repeated allocation-free call")
+    side = torch.cuda.Stream(gpu)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _capi.check("captured call", lib.mops_hip_attn_paged_decode_noalloc_bf16(*args, d["scale"], side.cuda_stream))
+    for i in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bit_exact(out, eager, f"replay {i} of the captured allocation-free call")
+
+
 def test_no_alloc_decode_rejects_what_does_not_fit(gpu):
     lib = _capi.load()
     A = 0x1000   # never dereferenced: the size check comes before any launch
