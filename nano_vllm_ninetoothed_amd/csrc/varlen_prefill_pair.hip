@@ -582,6 +582,17 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     else tile_barrier();
     if (ntiles <= 2 && tid < 64 && draw) park_ticket();
     int tile = 0;
+    // Steady prefix: tiles that lie below the diagonal of every wave of the item and whose successor is a whole tile (all
+    // but the item's last two).  Per tile two scalar additions, the tile, the barrier.
+    const int n_steady = min(ntiles - 2, cur.q0 >= 0 ? (cur.q0 + 1) / kPBN : 0);
+    for (; tile < n_steady; ++tile) {
+      kbase += kstep;
+      vbase += vstep;
+      tile_compute(tile, buf, kbase, vbase, std::false_type{}, std::false_type{}, 0, nullptr);
+      buf ^= 1;
+      item_barrier();   // the top of the next tile
+      if (tile == 0 && tid < 64 && draw) park_ticket();   // n_steady > 0 means more than two tiles
+    }
     for (; tile < ntiles - 1; ++tile) {
       kbase += kstep;
       vbase += vstep;
