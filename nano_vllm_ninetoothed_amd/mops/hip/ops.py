@@ -17,8 +17,20 @@ from ... import _capi
 from .registry import register_hip_op
 
 
+# The raw handle of the current stream of a device.  In the reference's own setting (eager, one Python call per op) the
+# host side of a decode step costs as much as its kernels, so the wrappers keep their per-call work small: this
+# lookup is 0.1 us where torch.cuda.current_stream(...).cuda_stream is 2 us, messages are only formatted on failure.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream_of(device: torch.device) -> int:
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 def _stream(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return _stream_of(t.device)
 
 
 def _require(cond: bool, msg: str) -> None:
@@ -27,8 +39,10 @@ def _require(cond: bool, msg: str) -> None:
 
 
 def _require_cuda_bf16(name: str, t: torch.Tensor) -> None:
-    _require(t.is_cuda, f"{name} must live on the GPU")
-    _require(t.dtype == torch.bfloat16, f"{name} must be bfloat16, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    if t.dtype != torch.bfloat16:
+        raise ValueError(f"{name} must be bfloat16, got {t.dtype}")
 
 
 # ----------------------------------------------------------------------------------------------------
@@ -129,15 +143,18 @@ def add_rms_forward(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tenso
     _require(x.shape == residual.shape, "x and residual must have the same shape")
     n = x.shape[-1]
     _require(weight.dim() == 1 and weight.shape[0] == n and weight.is_contiguous(), "weight must be [n] contiguous")
-    x2 = x.reshape(-1, n)
-    r2 = residual.reshape(-1, n)
+    x2 = x if x.dim() == 2 else x.reshape(-1, n)
+    r2 = residual if residual.dim() == 2 else residual.reshape(-1, n)
     if x2.stride(1) != 1:
         x2 = x2.contiguous()
     if r2.stride(1) != 1:
         r2 = r2.contiguous()
     rows = x2.shape[0]
-    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-    r_out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if x.is_contiguous():
+        y, r_out = torch.empty_like(x), torch.empty_like(x)
+    else:
+        y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        r_out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     lib = _capi.load()
     st = lib.mops_hip_add_rms_forward(x2.data_ptr(), x2.stride(0) if rows > 1 else n, r2.data_ptr(),
                                       r2.stride(0) if rows > 1 else n, weight.data_ptr(), y.data_ptr(),
@@ -152,8 +169,9 @@ _last_plan: dict = {}           # (device index, stream handle) -> description o
 
 
 def _workspace_key(device: torch.device):
-    return (device.index if device.index is not None else torch.cuda.current_device(),
-            torch.cuda.current_stream(device).cuda_stream)
+    if device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    return (device.index, _stream_of(device))
 
 
 def _decode_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
@@ -200,7 +218,8 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     HOLD what the planning call saw.  A caller that rewrites them in place (static graph buffers) and then passes
     reuse_plan=True without planning again gets the old split applied to the new lengths - truncated or zero rows,
     silently.  Plan once per decode step, as the engine counterpart does at layer 0."""
-    _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
+    if kwargs:
+        raise ValueError(f"unsupported arguments: {sorted(kwargs)}")
     _require(cache_seqlens is not None and block_table is not None, "cache_seqlens and block_table are required")
     _require_cuda_bf16("q", q)
     _require_cuda_bf16("k_cache", k_cache)
@@ -248,7 +267,8 @@ def flash_attn_varlen_func(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ma
     """Varlen causal prefill attention over packed [T, H, D] queries (call form: nanovllm/layers/attention.py:34-37).
     With block_table given, k and v are the paged caches and each sequence's keys are its cu_seqlens_k span
     (cached prefix + new tokens), masked bottom-right aligned."""
-    _require(not kwargs, f"unsupported arguments: {sorted(kwargs)}")
+    if kwargs:
+        raise ValueError(f"unsupported arguments: {sorted(kwargs)}")
     _require(causal, "only causal attention is implemented")
     _require(cu_seqlens_q is not None and max_seqlen_q is not None, "cu_seqlens_q and max_seqlen_q are required")
     _require_cuda_bf16("q", q)
@@ -308,7 +328,7 @@ _linear_pins_loaded = False
 
 
 def _linear_workspace(device: torch.device) -> torch.Tensor:
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    key = _workspace_key(device)
     ws = _linear_workspaces.get(key)
     if ws is None:
         ws = torch.empty(_LINEAR_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
