@@ -96,21 +96,26 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   __syncthreads();
   // Small launches also tabulate rank -> pair, a lookup per item instead of two searches: the thread that works out
   // from[l] knows where the pairs of q tile l - 1 start (at rank from[l]) and writes them down, sequences in order.
-  const bool tabulated = p.batch <= 64 && (p.total_tokens >> 6) + p.batch <= kPairTable;
+  const bool may_tabulate = p.batch <= 64 && (p.total_tokens >> 6) + p.batch <= kPairTable;
   for (int l = tid; l <= L.q_tiles + 1; l += kPThreads) {
     int s = 0;
     if (l < L.q_tiles)
       for (int b = 0; b < p.batch; ++b) s += max(0, t_cnt[b] - l);
     t_from[l] = s;
-    if (tabulated && l >= 1 && l <= L.q_tiles) {
+    if (may_tabulate && l >= 1 && l <= L.q_tiles) {
       for (int b = 0; b < p.batch; ++b)
-        if (t_cnt[b] > l - 1) t_pair[s++] = (b << 16) | (l - 1);
+        if (t_cnt[b] > l - 1) {
+          if (s < kPairTable) t_pair[s] = (b << 16) | (l - 1);
+          ++s;
+        }
     }
   }
   __syncthreads();
   const int home = (int)blockIdx.x % L.classes;   // the class this workgroup serves first
   const int member = (int)blockIdx.x / L.classes;
   const int n_pairs = __builtin_amdgcn_readfirstlane(t_from[0]);
+  // (offsets that are not non-decreasing can describe more pairs than the tokens allow for; the table is then not used)
+  const bool tabulated = may_tabulate && n_pairs <= kPairTable;
   const int n_items = n_pairs * L.units_per_class;   // items of a class (the same for all)
   if (tid == 0) t_tk[2] = home;
 
@@ -667,14 +672,20 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
       // item wait for its own output stores)
       asm volatile("" : "+v"(piece), "+v"(c4));
       uint16_t* const obase = p.out + (int64_t)(cur.seq_begin + wave_row0) * p.o_ts + (int64_t)(2 * cur.unit) * kPD + 8 * piece;
-      auto out_piece = [&](int i, auto all_rows) {
+      // all eight reads first, then the eight stores: written as read-store pairs, each store waited for its own read
+      u32x4 ow[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
         const int col = 4 * i + c4;           // column of the wave: head i >> 2, row col & 15
-        const int row = col & 15;
-        u32x4 w = *reinterpret_cast<const u32x4*>(stage + col * kPRow + ((piece ^ row) << 4));
-        if (i >= 4) w = u32x4{w[2], w[3], w[0], w[1]};
+        ow[i] = *reinterpret_cast<const u32x4*>(stage + col * kPRow + ((piece ^ (col & 15)) << 4));
+        if (i >= 4) ow[i] = u32x4{ow[i][2], ow[i][3], ow[i][0], ow[i][1]};
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      auto out_piece = [&](int i, auto all_rows) {
+        const int row = (4 * i + c4) & 15;
         // written once and not read again here: a streaming store leaves less for the write-back at the end of the kernel
         if (decltype(all_rows)::value || wave_row0 + row >= 0)
-          __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts + (i >> 2) * kPD));
+          __builtin_nontemporal_store(ow[i], reinterpret_cast<u32x4*>(obase + (int64_t)row * p.o_ts + (i >> 2) * kPD));
       };
       stores8 = __builtin_amdgcn_readfirstlane(wave_row0) >= 0;   // rows below 0 only exist in a sequence's first q tile
       if (stores8) {
