@@ -287,7 +287,7 @@ def main():
                                else "cfg2 varlen causal prefill, Qwen3-0.6B shape"), "batch": len(lens), "q_heads": 16, "kv_heads": 8,
                   "head_dim": 128, "seq_lens": "4 x 8192" if long_case else f"uniform[128,2048] seed {args.seed}",
                   "total_tokens": sum(lens)}
-        kernel_name = "varlen_prefill_kernel"
+        kernel_name = "varlen_prefill_pair_kernel<false>"
         if args.seed == 0:
             measured_traffic, traffic_source = profiled_traffic(args.op)
 
@@ -325,7 +325,7 @@ def main():
         config = {"workload": "varlen causal prefill behind a cached prefix, keys in the paged cache, Qwen3-0.6B shape", "batch": 16,
                   "q_heads": 16, "kv_heads": 8, "head_dim": 128, "new_tokens": "16 x 1024", "cached_prefix": "16 x 1024",
                   "block_size": W.BLOCK_SIZE}
-        kernel_name = "varlen_prefill_kernel"
+        kernel_name = "varlen_prefill_pair_kernel<true>"
 
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401

@@ -833,9 +833,10 @@ extern "C" int mops_hip_attn_varlen_causal_bf16(const void* q, int64_t q_token_s
   if (p.compact) pairs = pairs_bound;
   const int64_t grid = pairs * hq;
   if (grid > 0x7fffffffLL) return MOPS_HIP_EUNSUPPORTED;
-  // Grouped-query heads in pairs over the sequences' own keys take the form that packs two heads into a wave and keeps
-  // workgroups resident (varlen_prefill_pair.hip); everything else (cached prefix, paged caches, odd group sizes, very
-  // large batches, the form that scales Q once) stays here.  MOPS_HIP_PREFILL_FORM=rows forces this kernel.
+  // Grouped-query heads in pairs take the form that packs two heads into a wave and keeps workgroups resident
+  // (varlen_prefill_pair.hip), with or without a cached prefix; everything else (odd group sizes, very large batches, a
+  // cached prefix with more than 64 sequences or a block table of more than 768 entries, the form that scales Q once)
+  // stays here.  MOPS_HIP_PREFILL_FORM=rows forces this kernel.
   if (!prefill_prescale() && !prefill_force_rows()) {
     const int st = launch_prefill_pair(p, (hipStream_t)stream);
     if (st != MOPS_HIP_EUNSUPPORTED) return st;

@@ -1,6 +1,7 @@
-// Varlen (packed THD) causal prefill attention for gfx950, the form for grouped-query heads with an even group size and
-// keys that are the sequences' own tokens (no cached prefix): head_dim 128, bf16 MFMA for both products, fp32 online
-// softmax, K/V tiles staged through LDS.  The tile (blocks A, B, C, hand scheduled around the MFMAs) is the one of
+// Varlen (packed THD) causal prefill attention for gfx950, the form for grouped-query heads with an even group size:
+// head_dim 128, bf16 MFMA for both products, fp32 online softmax, K/V tiles staged through LDS.  Two instantiations: keys
+// that are the sequences' own tokens, and (PREFIX) keys behind a cached prefix, packed with offsets of their own or in the
+// paged caches, with the causal diagonal aligned bottom-right (query row i of a sequence sees keys 0 .. i + kv_len - len).  The tile (blocks A, B, C, hand scheduled around the MFMAs) is the one of
 // varlen_prefill.hip; what differs is what a wave's 32 MFMA columns are and how work reaches a workgroup.
 //
 // Work decomposition
@@ -31,6 +32,8 @@ constexpr int kPairMaxBatch = 512;     // sequences per launch (their offsets li
 constexpr int kPairMaxTiles = 1024;    // q tiles per sequence (65536 tokens)
 constexpr int kPairTable = 1024;       // (q tile, sequence) pairs whose rank -> pair mapping is tabulated in LDS
 constexpr int kPairSlots = 128;        // launches that may overlap on one device (one counter row each)
+constexpr int kPairPrefixBatch = 64;   // sequences per launch of the PREFIX form
+constexpr int kPairBlockEntries = 768; // block table entries (sequences x table width) the PREFIX form holds in LDS
 
 // Item counters, one row per slot: [c] next ticket of class c (the workgroups with id % classes == c), [8] workgroups
 // that have finished.  The last workgroup to finish zeroes its row, so a row is all zeros between launches.
@@ -44,6 +47,8 @@ struct PairLaunch {
   int members;          // workgroups per class
   int q_tiles;          // bound on the q tiles (64 rows) of a sequence
   int slot;             // counter row
+  int table_w;          // PREFIX, paged caches: block table entries per sequence held in LDS
+  int tiles_per_block;  // PREFIX, paged caches: 64-key tiles per cache block
 };
 
 // One 16-byte piece of the Q operand, loaded without the compiler knowing that the result arrives later: it then inserts
@@ -57,8 +62,13 @@ __device__ __forceinline__ void q_piece_async(bf16x8& dst, const char* ptr) {
 
 struct PairItem {
   int valid, seq_begin, seq_len, q0, unit, kv;   // unit: the head pair 2u, 2u + 1; kv: its kv head
+  // PREFIX: the sequence's keys.  kbegin: first key row (packed) or first entry of the sequence's block table in LDS (paged);
+  // kv_len: number of keys; shift = kv_len - seq_len: query row i sees keys 0 .. i + shift; steady: every cache block the
+  // item looks at exists
+  int kbegin, kv_len, shift, steady;
 };
 
+template <bool PREFIX>
 __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const PrefillParams p, const PairLaunch L) {
   // the factor between a score as the MFMA delivers it and the base-2 exponent (the sign of a negative scale is moved into Q)
   // (never exactly zero: a masked score is -inf, and -inf * 0 would be NaN where the probability has to be 0)
@@ -66,14 +76,19 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   // One array, so that the tile buffers start at the workgroup's LDS offset 0: a direct-to-LDS load takes its destination
   // from M0 as a plain offset.  K[2] then V[2] (16 KiB each), then the tables of the rank -> item mapping.
   constexpr int kTabCu = 0, kTabCnt = kPairMaxBatch + 4, kTabFrom = kTabCnt + kPairMaxBatch, kTabTicket = kTabFrom + kPairMaxTiles + 4,
-                kTabPair = kTabTicket + 4;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPTile + (kTabPair + kPairTable) * 4];
+                kTabPair = kTabTicket + 4, kTabCuK = kTabPair + kPairTable, kTabBlocks = kTabCuK + kPairPrefixBatch + 4,
+                kTabEnd = PREFIX ? kTabBlocks + kPairBlockEntries : kTabCuK;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPTile + kTabEnd * 4];
+  static_assert(2 * (4 * kPTile + kTabEnd * 4) <= 160 * 1024, "two workgroups per CU");
   int* const tab = reinterpret_cast<int*>(lds + 4 * kPTile);
   int* const t_cu = tab + kTabCu;        // cu_seqlens [batch + 1]
   int* const t_cnt = tab + kTabCnt;      // q tiles of sequence b
   int* const t_from = tab + kTabFrom;    // (q tile, sequence) pairs whose q tile index is >= l, l = 0 .. q_tiles + 1
   int* const t_pair = tab + kTabPair;    // pair of rank r as (sequence << 16 | q tile), when the launch is small enough for the table
   int* const t_tk = tab + kTabTicket;    // the ticket drawn during the current item
+  int* const t_cuk = tab + kTabCuK;      // PREFIX: cu_seqlens_k [batch + 1]
+  int* const t_bt = tab + kTabBlocks;    // PREFIX, paged: block table, table_w entries per sequence, -1 where there is no such block
+  const bool paged = PREFIX && p.block_table != nullptr;
   unsigned char* const lds_k = lds;
   unsigned char* const lds_v = lds + 2 * kPKTile;
 
@@ -87,6 +102,16 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
 
   // ---- tables of the rank -> item mapping (once per workgroup)
   for (int i = tid; i <= p.batch; i += kPThreads) t_cu[i] = p.cu_seqlens[i];
+  if (PREFIX) {
+    for (int i = tid; i <= p.batch; i += kPThreads) t_cuk[i] = p.cu_seqlens_k[i];
+    if (paged) {
+      for (int i = tid; i < p.batch * L.table_w; i += kPThreads) {
+        const int b = i / L.table_w;
+        const int e = p.block_table[(int64_t)b * p.block_table_row_stride + (i - b * L.table_w)];
+        t_bt[i] = (e >= 0 && e < p.num_blocks) ? e : -1;
+      }
+    }
+  }
   __syncthreads();
   for (int b = tid; b < p.batch; b += kPThreads) {
     const int qs = t_cu[b];
@@ -121,7 +146,7 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
 
   // rank (within the class, heaviest first) -> item.  Every wave works it out for itself; all values are wave-uniform.
   auto map_item = [&](int cls, int R) -> PairItem {
-    PairItem it = {0, 0, 0, 0, 0, 0};
+    PairItem it = {0, 0, 0, 0, 0, 0, 0, 0, 0, 1};
     if (R >= n_items) return it;
     // rank of the (q tile, sequence) pair and the head pair inside the class (no division for 1, 2, 4 .. pairs per class)
     const int pr = L.upc_shift >= 0 ? R >> L.upc_shift : R / L.units_per_class;
@@ -174,6 +199,25 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     it.q0 = __builtin_amdgcn_readfirstlane(seq_len - (seq_tiles - m) * kPairRows);
     it.unit = __builtin_amdgcn_readfirstlane(unit);
     it.kv = L.classes == 8 ? cls : it.unit / L.units_per_kv;
+    if (PREFIX) {
+      const int kb = t_cuk[b];
+      int kv_len = t_cuk[b + 1] - kb;
+      kv_len = min(kv_len, paged ? L.table_w * p.block_size : p.total_k_tokens - kb);
+      kv_len = kb >= 0 ? max(kv_len, 0) : 0;
+      it.kv_len = __builtin_amdgcn_readfirstlane(kv_len);
+      it.shift = it.kv_len - it.seq_len;
+      it.kbegin = __builtin_amdgcn_readfirstlane(paged ? b * L.table_w : kb);
+      if (paged) {
+        // whether every block under the keys the item looks at exists
+        const int kv_end = max(0, min(it.kv_len, it.q0 + kPairRows + it.shift));
+        const int used = (kv_end + p.block_size - 1) / p.block_size;
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        bool bad = false;
+        for (int j = 0; j < used; j += 64) bad |= (j + ln < used) && t_bt[it.kbegin + j + ln] < 0;
+        it.steady = __ballot(bad) == 0;
+      }
+    }
     return it;
   };
 
@@ -258,8 +302,29 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
       default: q_piece_async<224>(qb[7], ptr); break;
     }
   };
-  auto kv_base = [&](const PairItem& it, const uint16_t* base, int64_t ts) -> uint64_t {
-    return reinterpret_cast<uint64_t>(base) + (uint64_t)(((int64_t)it.seq_begin * ts + (int64_t)it.kv * kPD) * 2);
+  // Base addresses of an item's first K/V tile, and whether that tile holds a key the item looks at.  A tile that does
+  // not (no keys at all, a cache block that does not exist) is loaded from the start of the buffer, which is memory that
+  // exists, and not computed on.  PREFIX: k_ts / v_ts are the row strides of the keys, packed or inside a cache block.
+  const uint64_t block_bytes = PREFIX ? (uint64_t)p.block_size * (uint64_t)p.k_ts * 2u : 0u;
+  auto first_tile = [&](const PairItem& it, uint64_t& kb, uint64_t& vb) -> bool {
+    const uint64_t kroot = reinterpret_cast<uint64_t>(p.k) + (uint64_t)(it.kv * kPD * 2);
+    const uint64_t vroot = reinterpret_cast<uint64_t>(p.v) + (uint64_t)(it.kv * kPD * 2);
+    if (!PREFIX) {
+      kb = kroot + (uint64_t)((int64_t)it.seq_begin * p.k_ts * 2);
+      vb = vroot + (uint64_t)((int64_t)it.seq_begin * p.v_ts * 2);
+      return true;
+    }
+    bool ex = min(it.kv_len, it.q0 + kPairRows + it.shift) > 0;
+    if (paged) {
+      const int e = ex ? __builtin_amdgcn_readfirstlane(t_bt[it.kbegin]) : -1;
+      ex = e >= 0;
+      kb = kroot + (uint64_t)max(e, 0) * block_bytes;
+      vb = vroot + (uint64_t)max(e, 0) * block_bytes;
+    } else {
+      kb = kroot + (uint64_t)((int64_t)(ex ? it.kbegin : 0) * p.k_ts * 2);
+      vb = vroot + (uint64_t)((int64_t)(ex ? it.kbegin : 0) * p.v_ts * 2);
+    }
+    return ex;
   };
 
   // One tile, hand scheduled.  Every MFMA opens a slot; the instructions that follow it up to the next
@@ -498,10 +563,13 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   const uint64_t kstep = (uint64_t)kPBN * (uint64_t)p.k_ts * 2u, vstep = (uint64_t)kPBN * (uint64_t)p.v_ts * 2u;
   int clamp = 63;     // the last-row clamp ko / vo are set for
   int buf = 0;        // tile buffer pair the tile about to be computed sits in
+  bool tile_exists = true;   // PREFIX: whether the tile about to be computed holds keys (see first_tile)
   if (cur.valid) {
-    clamp = min(63, cur.seq_len - 1);
+    clamp = max(0, min(63, (PREFIX ? cur.kv_len : cur.seq_len) - 1));
     set_offsets(clamp);
-    loads_only(kv_base(cur, p.k, p.k_ts), kv_base(cur, p.v, p.v_ts), lds_s);
+    uint64_t kb0, vb0;
+    tile_exists = first_tile(cur, kb0, vb0);
+    loads_only(kb0, vb0, lds_s);
     const char* qa = q_address(cur);
 #pragma unroll
     for (int kb = 0; kb < 8; ++kb) q_load(kb, qa);
@@ -573,13 +641,39 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     m_run = -INFINITY;
     l_run = 0.f;
 
-    const int ntiles = (cur.q0 + kPairRows + kPBN - 1) / kPBN;      // K/V tiles the item looks at (keys 0 .. q0 + 63)
+    // query row i sees keys 0 .. i + shift, of kv_len keys (shift = 0 and kv_len = seq_len without a cached prefix)
+    const int shift = PREFIX ? cur.shift : 0;
+    const int kv_len = PREFIX ? cur.kv_len : cur.seq_len;
+    // K/V tiles the item looks at (keys 0 .. q0 + 63 + shift); an item that sees no key at all goes through one tile that
+    // nobody computes on
+    const int ntiles = PREFIX ? max(1, (min(kv_len, cur.q0 + kPairRows + shift) + kPBN - 1) / kPBN) : (cur.q0 + kPairRows + kPBN - 1) / kPBN;
     const int wave_row0 = cur.q0 + kPairWaveRows * wave;           // first q row (sequence-relative) of this wave
     const int my_row = wave_row0 + rloc;
+    const int wave_last = wave_row0 + kPairWaveRows - 1 + shift;   // last key the wave's last row sees
     // tiles this wave has to look at, and those of them that lie wholly below its first row's diagonal
-    const int my_tiles = wave_row0 + kPairWaveRows - 1 >= 0 ? min(ntiles, (wave_row0 + kPairWaveRows - 1) / kPBN + 1) : 0;
-    const int unmasked = wave_row0 >= 0 ? (wave_row0 + 1) / kPBN : 0;
-    uint64_t kbase = kv_base(cur, p.k, p.k_ts), vbase = kv_base(cur, p.v, p.v_ts);   // base of the tile after the one being computed
+    const int my_tiles = wave_last >= 0 ? min(ntiles, wave_last / kPBN + 1) : 0;
+    const int unmasked = wave_row0 + shift >= 0 ? (wave_row0 + shift + 1) / kPBN : 0;
+    uint64_t kbase, vbase;   // base of the tile after the one being computed
+    first_tile(cur, kbase, vbase);
+    // paged caches: block and tile inside the block of the tile kbase / vbase point at; whether that tile exists
+    int blk_i = 0, in_blk = 0;
+    bool next_exists = tile_exists;   // tiles of one block exist together
+    auto advance = [&]() {
+      if (paged) {
+        if (++in_blk == L.tiles_per_block) {
+          in_blk = 0;
+          ++blk_i;
+          const int e = __builtin_amdgcn_readfirstlane(t_bt[cur.kbegin + blk_i]);
+          next_exists = e >= 0;
+          const uint64_t off = (uint64_t)max(e, 0) * block_bytes + (uint64_t)(cur.kv * kPD * 2);
+          kbase = reinterpret_cast<uint64_t>(p.k) + off;
+          vbase = reinterpret_cast<uint64_t>(p.v) + off;
+          return;
+        }
+      }
+      kbase += kstep;
+      vbase += vstep;
+    };
     // The item's first barrier.  (Wave 0 has one or two more operations in flight, the draw and the look at the counters; eight
     // may stay in flight there too, which then makes it wait for as many stores.)  The ticket goes to LDS behind a barrier that has waited for the draw:
     // the second one, or, for items of one or two tiles, here, where the compiler puts the wait in front of the write.
@@ -589,28 +683,27 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     int tile = 0;
     // Steady prefix: tiles that lie below the diagonal of every wave of the item and whose successor is a whole tile (all
     // but the item's last two).  Per tile two scalar additions, the tile, the barrier.
-    const int n_steady = min(ntiles - 2, cur.q0 >= 0 ? (cur.q0 + 1) / kPBN : 0);
+    const int n_steady = (PREFIX && !cur.steady) ? 0 : min(ntiles - 2, cur.q0 + shift >= 0 ? (cur.q0 + shift + 1) / kPBN : 0);
     for (; tile < n_steady; ++tile) {
-      kbase += kstep;
-      vbase += vstep;
+      advance();
       tile_compute(tile, buf, kbase, vbase, std::false_type{}, std::false_type{}, 0, nullptr);
       buf ^= 1;
       item_barrier();   // the top of the next tile
       if (tile == 0 && tid < 64 && draw) park_ticket();   // n_steady > 0 means more than two tiles
     }
     for (; tile < ntiles - 1; ++tile) {
-      kbase += kstep;
-      vbase += vstep;
-      // the successor is a tile of this item; only the item's last tile can reach past the end of the sequence
-      const int want = min(63, cur.seq_len - 1 - (tile + 1) * kPBN);
+      advance();
+      // the successor is a tile of this item; only the item's last tile can reach past the end of the keys
+      const int want = min(63, kv_len - 1 - (tile + 1) * kPBN);
       if (want != clamp) {
         clamp = want;
         set_offsets(clamp);
       }
-      if (tile >= my_tiles) loads_only(kbase, vbase, lds_s + (unsigned)((buf ^ 1) * kPKTile));
+      if (tile >= my_tiles || (PREFIX && !tile_exists)) loads_only(kbase, vbase, lds_s + (unsigned)((buf ^ 1) * kPKTile));
       else if (tile < unmasked) tile_compute(tile, buf, kbase, vbase, std::false_type{}, std::false_type{}, 0, nullptr);
-      else if (wave_row0 + kPairWaveRows - 1 < tile * kPBN + 32) tile_compute_half(tile, buf, kbase, vbase, std::false_type{}, my_row, nullptr);
-      else tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::false_type{}, my_row, nullptr);
+      else if (wave_last < tile * kPBN + 32) tile_compute_half(tile, buf, kbase, vbase, std::false_type{}, my_row + shift, nullptr);
+      else tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::false_type{}, my_row + shift, nullptr);
+      if (PREFIX) tile_exists = next_exists;
       buf ^= 1;
       item_barrier();   // the top of the next tile
       if (tile == 0 && ntiles > 2 && tid < 64 && draw) park_ticket();
@@ -625,23 +718,23 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
         nxt = map_item(__builtin_amdgcn_readfirstlane(t_tk[1]), 2 * L.members + __builtin_amdgcn_readfirstlane(t_tk[0]));
       }
       const PairItem& to = nxt.valid ? nxt : cur;
-      kbase = kv_base(to, p.k, p.k_ts);
-      vbase = kv_base(to, p.v, p.v_ts);
-      const int want = min(63, to.seq_len - 1);
+      next_exists = first_tile(to, kbase, vbase);
+      const int want = max(0, min(63, (PREFIX ? to.kv_len : to.seq_len) - 1));
       if (want != clamp) {
         clamp = want;
         set_offsets(clamp);
       }
       const char* qnext = q_address(to);
-      if (tile >= my_tiles) {
+      if (tile >= my_tiles || (PREFIX && !tile_exists)) {
         loads_only(kbase, vbase, lds_s + (unsigned)((buf ^ 1) * kPKTile));
 #pragma unroll
         for (int kb = 0; kb < 8; ++kb) q_load(kb, qnext);
-      } else if (wave_row0 + kPairWaveRows - 1 < tile * kPBN + 32) {
-        tile_compute_half(tile, buf, kbase, vbase, std::true_type{}, my_row, qnext);
+      } else if (wave_last < tile * kPBN + 32) {
+        tile_compute_half(tile, buf, kbase, vbase, std::true_type{}, my_row + shift, qnext);
       } else {
-        tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::true_type{}, my_row, qnext);
+        tile_compute(tile, buf, kbase, vbase, std::true_type{}, std::true_type{}, my_row + shift, qnext);
       }
+      if (PREFIX) tile_exists = next_exists;
     }
     // Every wave is done with the last tile: its buffer pair is free for the epilogue.  Only LDS traffic is waited for:
     // the loads in flight are the next item's (into the other buffer pair and into qb), which the epilogue does not touch.
@@ -710,10 +803,24 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   }
 }
 
-int launch_prefill_pair(const PrefillParams& p, hipStream_t stream) {
-  if (p.block_table != nullptr || p.cu_seqlens_k != p.cu_seqlens || p.total_k_tokens != p.total_tokens) return MOPS_HIP_EUNSUPPORTED;
+int launch_prefill_pair(const PrefillParams& p_in, hipStream_t stream) {
+  PrefillParams p = p_in;
+  const bool paged = p.block_table != nullptr;
+  const bool prefix = paged || p.cu_seqlens_k != p.cu_seqlens || p.total_k_tokens != p.total_tokens;
   if (p.group < 2 || (p.group & 1) || p.batch > kPairMaxBatch) return MOPS_HIP_EUNSUPPORTED;
   PairLaunch L;
+  L.table_w = 0;
+  L.tiles_per_block = 1;
+  if (prefix) {
+    // the keys' offsets and the block table are held in LDS; launches too large for that take the other kernel
+    if (p.batch > kPairPrefixBatch || (!paged && p.total_k_tokens < 1)) return MOPS_HIP_EUNSUPPORTED;
+    if (paged) {
+      if ((int64_t)p.batch * p.max_blocks_per_seq > kPairBlockEntries || p.block_size % kPBN != 0) return MOPS_HIP_EUNSUPPORTED;
+      L.table_w = p.max_blocks_per_seq;
+      L.tiles_per_block = p.block_size / kPBN;
+      p.k_ts = p.v_ts = (int64_t)p.hkv * kPD;   // rows of a cache block
+    }
+  }
   // m_tiles counts 128-row tiles of the longest sequence; twice as many 64-row tiles bound it here
   L.q_tiles = 2 * p.m_tiles;
   if (L.q_tiles > kPairMaxTiles) return MOPS_HIP_EUNSUPPORTED;
@@ -737,7 +844,9 @@ int launch_prefill_pair(const PrefillParams& p, hipStream_t stream) {
   L.members = (int)std::min<int64_t>(items_bound, std::max(1, 2 * cus / L.classes));
   static std::atomic<unsigned> next_slot{0};
   L.slot = (int)(next_slot.fetch_add(1, std::memory_order_relaxed) % kPairSlots);
-  hipLaunchKernelGGL(varlen_prefill_pair_kernel, dim3((unsigned)(L.members * L.classes)), dim3(kPThreads), 0, stream, p, L);
+  const dim3 grid((unsigned)(L.members * L.classes));
+  if (prefix) hipLaunchKernelGGL(varlen_prefill_pair_kernel<true>, grid, dim3(kPThreads), 0, stream, p, L);
+  else hipLaunchKernelGGL(varlen_prefill_pair_kernel<false>, grid, dim3(kPThreads), 0, stream, p, L);
   return finish_launch();
 }
 

@@ -88,10 +88,10 @@ for qmul in (1.0, 4.0):
 
 
 def test_prefill_row_form_still_matches_oracle(gpu):
-    """Plain causal prefill over grouped heads takes the two-heads-per-wave form (varlen_prefill_pair.hip); the 128-row form
-    stays the path of cached prefixes, odd group sizes and very large batches.  MOPS_HIP_PREFILL_FORM=rows (read once per
-    process, hence the child process) forces it for plain inputs too, so that its ragged and rectangular launches stay
-    covered against the oracle."""
+    """Causal prefill over grouped heads takes the two-heads-per-wave form (varlen_prefill_pair.hip); the 128-row form
+    stays the path of odd group sizes, very large batches and block tables too large for LDS.  MOPS_HIP_PREFILL_FORM=rows
+    (read once per process, hence the child process) forces it for every input, so that its ragged and rectangular
+    launches and its paged and packed cached-prefix paths stay covered against the oracle."""
     import os, subprocess, sys
     code = r'''
 import sys, torch
@@ -108,13 +108,25 @@ for lens in ([300, 1, 77, 513], [256, 256], [2048], [0, 31, 700, 64, 65, 1, 129]
     w = ref(d["q"], d["k"], d["v"], max_seqlen_q=d["max_seqlen"], cu_seqlens_q=d["cu_seqlens"], softmax_scale=d["scale"]).float()
     e = (o - w).abs()
     print(len(lens), float(e.max()), float(e.mean()))
+for new, prefix in (([100, 200], [256, 512]), ([300, 17, 129], [0, 256, 768]), ([1, 1, 1], [256, 1, 1023]), ([200], [17000])):
+    d = W.prefix_prefill_inputs(new, prefix, seed=sum(new) + sum(prefix))
+    g = W.to_device(d, dev)
+    w = ref(d["q"], torch.nan_to_num(d["k_cache"]), torch.nan_to_num(d["v_cache"]), max_seqlen_q=d["max_seqlen_q"],
+            cu_seqlens_q=d["cu_seqlens_q"], max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"],
+            softmax_scale=d["scale"], causal=True, block_table=d["block_table"]).float()
+    for paged in (True, False):
+        k, v = (g["k_cache"], g["v_cache"]) if paged else (g["k_all"], g["v_all"])
+        o = hip(g["q"], k, v, max_seqlen_q=d["max_seqlen_q"], cu_seqlens_q=g["cu_seqlens_q"], max_seqlen_k=d["max_seqlen_k"],
+                cu_seqlens_k=g["cu_seqlens_k"], softmax_scale=d["scale"], causal=True, block_table=g["block_table"] if paged else None).cpu().float()
+        e = (o - w).abs()
+        print(len(new), float(e.max()), float(e.mean()))
 ''' % (gpu.index or 0)
     env = dict(os.environ, MOPS_HIP_PREFILL_FORM="rows")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=150)
     assert out.returncode == 0, out.stderr[-2000:]
-    rows = [l.split() for l in out.stdout.strip().splitlines()[-4:]]
-    assert len(rows) == 4
+    rows = [l.split() for l in out.stdout.strip().splitlines()[-12:]]
+    assert len(rows) == 12
     for n, mx, mean in rows:
         assert float(mx) <= 2e-2 and float(mean) <= 2e-3, (n, mx, mean)
 
@@ -284,6 +296,39 @@ def test_prefill_with_cached_prefix_other_block_sizes_and_long_tables(gpu, ops, 
     got = _run_prefix(hip, d, gpu, paged=True)
     assert_attention_close(got, want, f"paged prefix prefill, block size {block_size}, new={new} prefix={prefix}")
     assert_bit_exact(_run_prefix(hip, d, gpu, paged=False), got, "packed keys with cu_seqlens_k vs paged keys")
+
+
+def test_prefix_prefill_with_a_block_table_too_large_for_the_resident_form(gpu, ops):
+    """The two-heads-per-wave form keeps the block table in LDS (768 entries); 40 sequences x 24 blocks do not fit and go
+    to the 128-row form, as do more than 64 sequences with a prefix."""
+    hip, ref = ops("flash_attn_varlen_func")
+    for new, prefix in (([20, 70] * 20, [6000, 300] * 20), ([5] * 70, [300] * 70)):
+        d = W.prefix_prefill_inputs(new, prefix, hq=4, hkv=2, seed=len(new))
+        assert len(new) > 64 or d["block_table"].numel() > 768
+        want = ref(d["q"], torch.nan_to_num(d["k_cache"]), torch.nan_to_num(d["v_cache"]), max_seqlen_q=d["max_seqlen_q"],
+                   cu_seqlens_q=d["cu_seqlens_q"], max_seqlen_k=d["max_seqlen_k"], cu_seqlens_k=d["cu_seqlens_k"],
+                   softmax_scale=d["scale"], causal=True, block_table=d["block_table"])
+        assert_attention_close(_run_prefix(hip, d, gpu, paged=True), want, f"paged prefix prefill, {len(new)} sequences")
+
+
+def test_prefix_prefill_sequence_without_keys_gives_zeros(gpu, ops):
+    """cu_seqlens_k may give a sequence no keys at all, or fewer keys than queries (rows whose horizon lies before key 0
+    see nothing): such rows come out as zeros, the other sequences are not disturbed."""
+    hip, ref = ops("flash_attn_varlen_func")
+    d = W.prefix_prefill_inputs([50, 100, 70], [0, 200, 0], seed=77)
+    g = W.to_device(d, gpu)
+    # sequence 0 keeps no keys; sequence 2 keeps 30 keys for its 70 queries: rows 0..39 see nothing, row 40 + i sees keys 0..i
+    cu_k = torch.tensor([0, 0, 300, 330], dtype=torch.int32)
+    got = hip(g["q"], g["k_all"][50:], g["v_all"][50:], max_seqlen_q=100, cu_seqlens_q=g["cu_seqlens_q"], max_seqlen_k=300,
+              cu_seqlens_k=cu_k.to(gpu), softmax_scale=d["scale"], causal=True).cpu()
+    assert torch.isfinite(got.float()).all()
+    assert (got[:50] == 0).all() and (got[150:190] == 0).all()
+    want1 = ref(d["q"][50:150], d["k_all"][50:350], d["v_all"][50:350], max_seqlen_q=100, cu_seqlens_q=torch.tensor([0, 100], dtype=torch.int32),
+                max_seqlen_k=300, cu_seqlens_k=torch.tensor([0, 300], dtype=torch.int32), softmax_scale=d["scale"], causal=True)
+    assert_attention_close(got[50:150], want1, "sequence between two sequences without visible keys")
+    want2 = ref(d["q"][190:220], d["k_all"][350:380], d["v_all"][350:380], max_seqlen_q=30, cu_seqlens_q=torch.tensor([0, 30], dtype=torch.int32),
+                max_seqlen_k=30, cu_seqlens_k=torch.tensor([0, 30], dtype=torch.int32), softmax_scale=d["scale"], causal=True)
+    assert_attention_close(got[190:220], want2, "the rows of a sequence with fewer keys than queries that do see keys")
 
 
 def test_prefix_prefill_treats_a_missing_block_as_empty(gpu, ops):
