@@ -57,7 +57,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 50; 500 for the prefill ops)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed warm-up steps (default 10; 300 for the prefill ops)")
     ap.add_argument("--op", default="decode",
-                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "store", "silu", "sampler", "qk_rope_store", "add_rms", "rms", "embedding", "copy", "launch_floor", "e2e"])
+                    choices=["decode", "decode8b", "prefill", "prefill_long", "prefix_prefill", "prefix_prefill_short", "store", "silu", "sampler", "qk_rope_store", "add_rms", "rms", "embedding", "copy", "launch_floor", "e2e"])
     ap.add_argument("--e2e-seqs", type=int, default=256, help="number of prompts of the e2e workload")
     ap.add_argument("--e2e-eager", action="store_true", help="e2e: no HIP-graph replay of the decode step")
     ap.add_argument("--e2e-stepwise", action="store_true", help="e2e: read every step's tokens back before the next step, as the reference does")
@@ -69,7 +69,7 @@ def parse_args():
     # to that load with a transient: launches 10..150 of a back-to-back series run up to 40 % slower than the first ten
     # and than everything after launch 250.  The warm-up of these ops is long enough to sit the transient out, and the
     # timed series long enough not to be dominated by what is left of it.
-    matrix_bound = args.op in ("prefill", "prefill_long", "prefix_prefill")
+    matrix_bound = args.op in ("prefill", "prefill_long", "prefix_prefill", "prefix_prefill_short")
     if args.steps is None:
         args.steps = 500 if matrix_bound else 50
     if args.warmup is None:
@@ -307,10 +307,12 @@ def main():
                 ts.append(time.perf_counter() - t0)
             return sorted(ts)[1], "whole batch, median of 3", work
 
-    elif args.op == "prefix_prefill":
+    elif args.op in ("prefix_prefill", "prefix_prefill_short"):
         # prefix-cache hit (nanovllm/layers/attention.py:32-33 of the reference): 16 sequences with 1024 tokens already in
-        # the paged cache and 1024 new ones; keys are read through block_table
-        new, prefix = [1024] * 16, [1024] * 16
+        # the paged cache and 1024 new ones; keys are read through block_table.  The short case is the shape of a shared
+        # prompt followed by a few new tokens: 32 sequences, 2048 cached and 64 new tokens each.
+        short_case = args.op == "prefix_prefill_short"
+        new, prefix = ([64] * 32, [2048] * 32) if short_case else ([1024] * 16, [1024] * 16)
         d = W.to_device(W.prefix_prefill_inputs(new, prefix, seed=args.seed, poison_unused=False), dev)
         op = mops.flash_attn_varlen_func
 
@@ -322,19 +324,20 @@ def main():
         work = float(sum(4 * 128 * 16 * (n * pl + n * (n + 1) // 2) for n, pl in zip(new, prefix)))
         bound = "mfma"
         metric, unit = "varlen_prefill_attn_TFLOPs", "TFLOP/s"
-        config = {"workload": "varlen causal prefill behind a cached prefix, keys in the paged cache, Qwen3-0.6B shape", "batch": 16,
-                  "q_heads": 16, "kv_heads": 8, "head_dim": 128, "new_tokens": "16 x 1024", "cached_prefix": "16 x 1024",
-                  "block_size": W.BLOCK_SIZE}
-        kernel_name = "varlen_prefill_pair_kernel<true>"
+        config = {"workload": "varlen causal prefill behind a cached prefix, keys in the paged cache, Qwen3-0.6B shape", "batch": len(new),
+                  "q_heads": 16, "kv_heads": 8, "head_dim": 128, "new_tokens": f"{len(new)} x {new[0]}",
+                  "cached_prefix": f"{len(new)} x {prefix[0]}", "block_size": W.BLOCK_SIZE}
+        # long runs of new tokens stay on the 128-row kernel, few new tokens per sequence take the two-heads-per-wave form
+        kernel_name = "varlen_prefill_pair_kernel<true>" if short_case else "varlen_prefill_kernel<false>"
 
         def cpu_fn():
             import oracle.mops_torch  # noqa: F401
             ref = mops.get_op("flash_attn_varlen_func", "torch")
             c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
             t0 = time.perf_counter()
-            ref(c["q"][:1024], c["k_cache"], c["v_cache"], max_seqlen_q=1024, cu_seqlens_q=c["cu_seqlens_q"][:2], max_seqlen_k=2048,
+            ref(c["q"][:new[0]], c["k_cache"], c["v_cache"], max_seqlen_q=new[0], cu_seqlens_q=c["cu_seqlens_q"][:2], max_seqlen_k=new[0] + prefix[0],
                 cu_seqlens_k=c["cu_seqlens_k"][:2], softmax_scale=c["scale"], causal=True, block_table=c["block_table"][:1])
-            return time.perf_counter() - t0, "first of the 16 sequences, one run", work / 16
+            return time.perf_counter() - t0, f"first of the {len(new)} sequences, one run", work / len(new)
 
     elif args.op == "store":
         lens = W.random_seq_lens(16, 128, 2048, seed=args.seed)
@@ -597,7 +600,7 @@ def main():
         cval = units / secs / (1e9 if bound == "hbm" else 1e12)
         out["cpu_baseline"] = {"value": round(cval, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
                                "sample": sample, "seconds": round(secs, 4)}
-    if args.op in ("prefill", "prefill_long", "prefix_prefill"):
+    if args.op in ("prefill", "prefill_long", "prefix_prefill", "prefix_prefill_short"):
         # what a library bf16 GEMM sustains on this chip in this run: the 2.5 PFLOP/s peak assumes 2.4 GHz, which the
         # part does not hold under matrix load, so this is the practical MFMA ceiling to read the fraction against
         n = 8192

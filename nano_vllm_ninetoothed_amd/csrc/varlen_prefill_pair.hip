@@ -101,7 +101,18 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
   const int rloc = n & 15;    // its row inside the wave's 16 rows
 
   // ---- tables of the rank -> item mapping (once per workgroup)
-  for (int i = tid; i <= p.batch; i += kPThreads) t_cu[i] = p.cu_seqlens[i];
+  // (a thread takes both offsets of its sequence from memory: the q tile counts need no second pass over LDS)
+  for (int b = tid; b < ((p.batch + 15) & ~15); b += kPThreads) {
+    int cnt = 0;
+    if (b < p.batch) {
+      const int qs = p.cu_seqlens[b], qe = p.cu_seqlens[b + 1];
+      t_cu[b] = qs;
+      if (b == p.batch - 1) t_cu[p.batch] = qe;
+      const int len = min(qe, p.total_tokens) - qs;
+      cnt = (qs >= 0 && len > 0) ? min((len + kPairRows - 1) / kPairRows, L.q_tiles) : 0;
+    }
+    t_cnt[b] = cnt;   // zero up to a multiple of 16: the passes below read the counts sixteen at a time
+  }
   if (PREFIX) {
     for (int i = tid; i <= p.batch; i += kPThreads) t_cuk[i] = p.cu_seqlens_k[i];
     if (paged) {
@@ -113,26 +124,30 @@ __global__ __launch_bounds__(kPThreads, 2) void varlen_prefill_pair_kernel(const
     }
   }
   __syncthreads();
-  for (int b = tid; b < p.batch; b += kPThreads) {
-    const int qs = t_cu[b];
-    const int len = min(t_cu[b + 1], p.total_tokens) - qs;
-    t_cnt[b] = (qs >= 0 && len > 0) ? min((len + kPairRows - 1) / kPairRows, L.q_tiles) : 0;
-  }
-  __syncthreads();
   // Small launches also tabulate rank -> pair, a lookup per item instead of two searches: the thread that works out
   // from[l] knows where the pairs of q tile l - 1 start (at rank from[l]) and writes them down, sequences in order.
   const bool may_tabulate = p.batch <= 64 && (p.total_tokens >> 6) + p.batch <= kPairTable;
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+  const i32x4* const cnt4 = reinterpret_cast<const i32x4*>(t_cnt);
   for (int l = tid; l <= L.q_tiles + 1; l += kPThreads) {
     int s = 0;
     if (l < L.q_tiles)
-      for (int b = 0; b < p.batch; ++b) s += max(0, t_cnt[b] - l);
+      for (int b = 0; b < p.batch; b += 16) {
+        const i32x4 c0 = cnt4[b >> 2], c1 = cnt4[(b >> 2) + 1], c2 = cnt4[(b >> 2) + 2], c3 = cnt4[(b >> 2) + 3];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s += max(0, c0[e] - l) + max(0, c1[e] - l) + max(0, c2[e] - l) + max(0, c3[e] - l);
+      }
     t_from[l] = s;
     if (may_tabulate && l >= 1 && l <= L.q_tiles) {
-      for (int b = 0; b < p.batch; ++b)
-        if (t_cnt[b] > l - 1) {
-          if (s < kPairTable) t_pair[s] = (b << 16) | (l - 1);
-          ++s;
-        }
+      for (int b = 0; b < p.batch; b += 16) {
+        const i32x4 c[4] = {cnt4[b >> 2], cnt4[(b >> 2) + 1], cnt4[(b >> 2) + 2], cnt4[(b >> 2) + 3]};
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          if (c[e >> 2][e & 3] > l - 1) {
+            if (s < kPairTable) t_pair[s] = ((b + e) << 16) | (l - 1);
+            ++s;
+          }
+      }
     }
   }
   __syncthreads();
@@ -814,6 +829,10 @@ int launch_prefill_pair(const PrefillParams& p_in, hipStream_t stream) {
   if (prefix) {
     // the keys' offsets and the block table are held in LDS; launches too large for that take the other kernel
     if (p.batch > kPairPrefixBatch || (!paged && p.total_k_tokens < 1)) return MOPS_HIP_EUNSUPPORTED;
+    // Behind a prefix every item is long, so what this form saves per item and on the diagonal is little; what remains is
+    // its finer q tiles (64 rows instead of 128), which pay when sequences bring few new tokens.  With long runs of new
+    // tokens the other kernel is the faster one in a sustained series of launches (16 x (1024 + 1024): by 2 %).
+    if ((int64_t)p.total_tokens > 512 * (int64_t)p.batch) return MOPS_HIP_EUNSUPPORTED;
     if (paged) {
       if ((int64_t)p.batch * p.max_blocks_per_seq > kPairBlockEntries || p.block_size % kPBN != 0) return MOPS_HIP_EUNSUPPORTED;
       L.table_w = p.max_blocks_per_seq;
