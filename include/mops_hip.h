@@ -213,8 +213,10 @@ int mops_hip_attn_paged_decode_noalloc_bf16(const void* q, int64_t q_batch_strid
  * (softmax_scale 128^-1/2 on N(0,1) data: outputs below 2, one bf16 ulp <= 0.0156).  The bound is one bf16 ulp of the
  * output, so it scales with the outputs: at softmax_scale 1 on the same data the outputs reach 4 (ulp 0.031) and the
  * tests allow max-abs 4e-2 there.
- * Launches with block_table == NULL, keys that are the sequences' own tokens, an even hq / hkv, up to 512 sequences and
- * up to 65536 tokens per sequence keep two workgroups per CU resident and hand them work items through counters in a
+ * Launches with an even hq / hkv, up to 512 sequences and up to 65536 tokens per sequence whose keys are the sequences'
+ * own tokens, and launches behind a cached prefix (cu_seqlens_k or block_table given) with at most 64 sequences, at
+ * most 512 new tokens per sequence on average and, when paged, at most 768 block table entries
+ * (batch * max_blocks_per_seq), keep two workgroups per CU resident and hand them work items through counters in a
  * device array inside the library (128 rows, one per launch, round robin, cleared by the launch): at most 128 such
  * launches may be in flight per device; a launch captured into a HIP graph keeps its row.  MOPS_HIP_PREFILL_FORM=rows
  * (read at the first call) keeps every launch on the one-workgroup-per-128-rows form the other inputs take.
