@@ -137,64 +137,146 @@ namespace mops {
 
 constexpr int kArgmaxThreads = 1024;
 
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+// One workgroup per row, in two passes.  Pass 1 streams the row once and keeps three running values per lane and 16-bit
+// half, over the raw bf16 bit patterns: their maximum and minimum as signed integers and their maximum as unsigned ones,
+// three packed instructions per two logits (comparing widened values with an index kept beside the maximum took twelve,
+// and at this size the kernel was as much instruction- as memory-bound).  Non-negative numbers order like their patterns
+// read as signed integers and lie above all negative ones, so a signed maximum >= 0 is the row's maximum; when it is
+// negative every logit is, negative numbers order against their patterns, and the signed minimum is the row's maximum.
+// The unsigned maximum is the negative pattern of largest magnitude when there is one: above 0xff80 it is a NaN.
+// Pass 2 finds the first index of the row maximum: only lanes whose own maximum equals it look again, at the one batch of
+// pieces in which their maximum first appeared (noted in pass 1 at the price of a few instructions per batch), which is
+// still in the L2.
+__device__ __forceinline__ float bits_to_f32(int b) { return __uint_as_float((unsigned)b << 16); }
+
 __global__ __launch_bounds__(kArgmaxThreads) void row_argmax_kernel(const uint16_t* __restrict__ logits, int64_t row_stride,
                                                                    int64_t* __restrict__ out, int n) {
-  __shared__ float best_v[kArgmaxThreads / kWave];
-  __shared__ int best_i[kArgmaxThreads / kWave];
-  __shared__ int spoiled_w[kArgmaxThreads / kWave];
+  __shared__ int smax_w[kArgmaxThreads / kWave], smin_w[kArgmaxThreads / kWave], umax_w[kArgmaxThreads / kWave];
+  __shared__ int first_i;
   const uint16_t* row = logits + (int64_t)blockIdx.x * row_stride;
-  float bv = -INFINITY;
-  int bi = 0x7fffffff;
-  // A NaN or +inf logit turns the whole softmax row into NaN, and the library's argmax of an all-NaN row is 0.
-  bool spoiled = false;
+  s16x2 smax2 = {(short)-32768, (short)-32768}, smin2 = {(short)32767, (short)32767};
+  u16x2 umax2 = {0, 0};
   const int pieces = n >> 3;
-  auto take = [&](const u32x4 w, int pc) {
+  auto take = [&](const u32x4 w) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float lo = bf16lo_to_f32(w[e]), hi = bf16hi_to_f32(w[e]);
-      const int i0 = (pc << 3) + 2 * e;
-      spoiled |= !(lo < INFINITY) || !(hi < INFINITY);
-      if (lo > bv) { bv = lo; bi = i0; }        // strictly greater: within a lane indices only grow
-      if (hi > bv) { bv = hi; bi = i0 + 1; }
+      // (a copy of the element first: a bit cast applied to the vector's element directly reads element 0 whatever e is)
+      const uint32_t d = w[e];
+      smax2 = __builtin_elementwise_max(smax2, __builtin_bit_cast(s16x2, d));
+      smin2 = __builtin_elementwise_min(smin2, __builtin_bit_cast(s16x2, d));
+      umax2 = __builtin_elementwise_max(umax2, __builtin_bit_cast(u16x2, d));
     }
   };
-  // four loads in flight per lane (eight are slower again): one workgroup per row leaves the memory system too little to do otherwise
-  constexpr int kDeep = 4;
+  // The lane's maximum so far as a score that grows with the number: the pattern itself when there is a non-negative
+  // logit, else below zero and falling with the signed minimum.  `at_pc`, `at_cnt`: the batch in which the score last
+  // grew, i.e. in which the lane's maximum first appeared (its first piece, its number of pieces; 0 pieces: the tail).
+  int smax = -32768, smin = 32767, score = -0x7fffffff, at_pc = 0, at_cnt = 0;
+  auto score_of = [](int mx, int mn) { return mx >= 0 ? mx : -1 - (mn + 32768); };
+  auto note = [&](int pc0, int cnt) {
+    smax = max((int)smax2[0], (int)smax2[1]);
+    smin = min((int)smin2[0], (int)smin2[1]);
+    const int sc = score_of(smax, smin);
+    if (sc > score) {
+      score = sc;
+      at_pc = pc0;
+      at_cnt = cnt;
+    }
+  };
+  // two loads in flight per lane (four and eight are slower): one workgroup per row leaves the memory system too little to do otherwise
+  constexpr int kDeep = 2;
   int pc = threadIdx.x;
   for (; pc + (kDeep - 1) * kArgmaxThreads < pieces; pc += kDeep * kArgmaxThreads) {
     u32x4 w[kDeep];
 #pragma unroll
     for (int u = 0; u < kDeep; ++u) w[u] = load16_stream(row + ((int64_t)(pc + u * kArgmaxThreads) << 3));
 #pragma unroll
-    for (int u = 0; u < kDeep; ++u) take(w[u], pc + u * kArgmaxThreads);
+    for (int u = 0; u < kDeep; ++u) take(w[u]);
+    note(pc, kDeep);
   }
-  for (; pc < pieces; pc += kArgmaxThreads) take(load16_stream(row + ((int64_t)pc << 3)), pc);
+  for (; pc < pieces; pc += kArgmaxThreads) {
+    take(load16_stream(row + ((int64_t)pc << 3)));
+    note(pc, 1);
+  }
+  int umax = max((int)umax2[0], (int)umax2[1]);
   for (int i = (pieces << 3) + threadIdx.x; i < n; i += kArgmaxThreads) {  // tail when n % 8 != 0
-    const float x = bf16lo_to_f32(row[i]);
-    spoiled |= !(x < INFINITY);
-    if (x > bv) { bv = x; bi = i; }
+    const int x = (int)(short)row[i];
+    smax = max(smax, x);
+    smin = min(smin, x);
+    umax = max(umax, x & 0xffff);
+    const int sc = score_of(smax, smin);
+    if (sc > score) {
+      score = sc;
+      at_cnt = 0;
+    }
   }
-  // an all -inf row is all NaN after the softmax as well: bi stays unset and becomes 0 below
+  const int lane_smax = smax, lane_smin = smin;
 #pragma unroll
   for (int off = kWave / 2; off >= 1; off >>= 1) {
-    const float ov = __shfl_xor(bv, off, kWave);
-    const int oi = __shfl_xor(bi, off, kWave);
-    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    smax = max(smax, __shfl_xor(smax, off, kWave));
+    smin = min(smin, __shfl_xor(smin, off, kWave));
+    umax = max(umax, __shfl_xor(umax, off, kWave));
   }
   if ((threadIdx.x & (kWave - 1)) == 0) {
-    best_v[threadIdx.x / kWave] = bv;
-    best_i[threadIdx.x / kWave] = bi;
+    smax_w[threadIdx.x / kWave] = smax;
+    smin_w[threadIdx.x / kWave] = smin;
+    umax_w[threadIdx.x / kWave] = umax;
   }
-  const bool wave_spoiled = __any(spoiled);
-  if ((threadIdx.x & (kWave - 1)) == 0) spoiled_w[threadIdx.x / kWave] = wave_spoiled;
+  if (threadIdx.x == 0) first_i = 0x7fffffff;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < kArgmaxThreads / kWave; ++w)
-      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
-    bool any_spoiled = false;
-    for (int w = 0; w < kArgmaxThreads / kWave; ++w) any_spoiled |= spoiled_w[w] != 0;
-    out[blockIdx.x] = (bi == 0x7fffffff || any_spoiled) ? 0 : bi;
+#pragma unroll
+  for (int w = 0; w < kArgmaxThreads / kWave; ++w) {
+    smax = max(smax, smax_w[w]);
+    smin = min(smin, smin_w[w]);
+    umax = max(umax, umax_w[w]);
   }
+  // A NaN or +inf logit turns the whole softmax row into NaN, and so does a row of -inf; the library's argmax of an
+  // all-NaN row is 0.  Patterns: +inf 0x7f80, NaNs above it; -inf 0xff80 (-128 as a signed value), NaNs above it.
+  const bool spoiled = smax >= 0x7f80 || umax > 0xff80 || (smax < 0 && smin >= -128) || smin > smax;
+  if (spoiled) {
+    if (threadIdx.x == 0) out[blockIdx.x] = 0;
+    return;
+  }
+  const float gv = bits_to_f32(smax >= 0 ? smax : smin);
+  // the lane's own maximum as a number (lanes that read nothing say -inf, which a row that got here does not have as its maximum)
+  const float lane_v = lane_smin > lane_smax ? -INFINITY : bits_to_f32(lane_smax >= 0 ? lane_smax : lane_smin);
+  // pass 2 (numbers compared as numbers: -0 and +0 tie, the first of them wins, as in the library)
+  if (__any(lane_v == gv)) {
+    int bi = 0x7fffffff;
+    if (lane_v == gv) {
+      // -0 and +0 are one number with two patterns: a lane that met -0 first and +0 later noted the later batch, so zeros
+      // are looked for from the lane's first piece on
+      const bool zero = gv == 0.f;
+      const int q0 = zero ? (int)threadIdx.x : at_pc;
+      const int q1 = zero ? pieces : (at_cnt == 0 ? 0 : min(pieces, at_pc + at_cnt * kArgmaxThreads));
+      for (int q = q0; q < q1 && bi == 0x7fffffff; q += kDeep * kArgmaxThreads) {
+        u32x4 w[kDeep];
+#pragma unroll
+        for (int u = 0; u < kDeep; ++u) {
+          const int qq = q + u * kArgmaxThreads;
+          w[u] = qq < q1 ? load16(row + ((int64_t)qq << 3)) : u32x4{0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};   // NaNs match nothing
+        }
+#pragma unroll
+        for (int u = kDeep - 1; u >= 0; --u)
+#pragma unroll
+          for (int e = 3; e >= 0; --e) {
+            const int i0 = ((q + u * kArgmaxThreads) << 3) + 2 * e;
+            if (bf16hi_to_f32(w[u][e]) == gv) bi = i0 + 1;
+            if (bf16lo_to_f32(w[u][e]) == gv) bi = i0;
+          }
+      }
+      if (bi == 0x7fffffff)
+        for (int i = (pieces << 3) + threadIdx.x; i < n && bi == 0x7fffffff; i += kArgmaxThreads)
+          if (bf16lo_to_f32(row[i]) == gv) bi = i;
+    }
+#pragma unroll
+    for (int off = kWave / 2; off >= 1; off >>= 1) bi = min(bi, __shfl_xor(bi, off, kWave));
+    if ((threadIdx.x & (kWave - 1)) == 0) atomicMin(&first_i, bi);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = first_i == 0x7fffffff ? 0 : first_i;
 }
 
 }  // namespace mops

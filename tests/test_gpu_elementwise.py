@@ -89,6 +89,39 @@ def test_sampler_on_rows_the_softmax_turns_into_nans(gpu, ops):
     assert got[:4].tolist() == [0, 0, 0, 0] and int(got[4]) == 1234
 
 
+def test_sampler_rows_of_negative_logits_zeros_of_both_signs_and_short_rows(gpu, ops):
+    """The kernel orders raw bf16 patterns: rows without a non-negative logit take the other branch of that order, -0 and
+    +0 are one number with two patterns (the first of either wins), negative NaNs and -inf sit at the far end of the
+    unsigned order, and a row may be shorter than one 16-byte piece or end in a partial one that holds the maximum."""
+    hip, ref = ops("sampler_forward")
+    g = torch.Generator().manual_seed(5)
+    n = 8 * 1024 * 5 + 3                                   # five pieces per lane and a tail of three
+    base = -(torch.rand((12, n), generator=g) * 20 + 0.5).to(torch.bfloat16)   # every logit negative
+    logits = base.clone()
+    logits[0, 4097] = -0.25                                # a row of negatives: the maximum is the smallest magnitude
+    logits[1, 77] = -0.0                                   # -0 is the maximum of a negative row
+    logits[2, 900] = 0.0; logits[2, 30] = -0.0            # -0 first, +0 later: one number, index 30
+    logits[3, 30] = 0.0; logits[3, 900] = -0.0
+    logits[4, n - 1] = 3.0                                 # the maximum in the partial last piece
+    logits[5, n - 2] = -0.125                              # the same in a negative row
+    logits[6, 10] = float("-inf"); logits[6, 4000] = -0.375
+    logits[7, 123] = torch.tensor(-float("nan"))           # a NaN with the sign bit set
+    logits[8, 5] = 7.0; logits[8, 2053] = 7.0; logits[8, 8192 * 3 + 5] = 7.0   # a tie across lanes and batches: the first wins
+    logits[9, 3000] = 1e-38                                # a tiny positive among negatives
+    logits[10, :] = -3.0                                   # all equal: index 0
+    logits[11, 1024 * 8 * 2 + 5] = 0.5; logits[11, 5] = 0.25   # same lane, later batch holds the maximum
+    temps = torch.full((12,), 0.7)
+    want = ref(logits, temps)
+    got = hip(logits.to(gpu), temps.to(gpu)).cpu()
+    assert torch.equal(got, want), (got.tolist(), want.tolist())
+    assert got.tolist()[:7] == [4097, 77, 30, 30, n - 1, n - 2, 4000] and int(got[7]) == 0 and int(got[8]) == 5
+    for width in (1, 3, 7, 8, 9):
+        small = (torch.randn((4, 16), generator=g) * 2).to(torch.bfloat16)
+        t4 = torch.full((4,), 0.7)
+        view = small[:, :width]
+        assert torch.equal(hip(small.to(gpu)[:, :width], t4.to(gpu)).cpu(), ref(view, t4)), width
+
+
 @pytest.mark.parametrize("tokens,hq,hkv,need_k", [(1, 16, 8, True), (5, 16, 8, False), (300, 16, 8, True), (64, 32, 8, False), (33, 8, 1, True)])
 def test_fused_qk_norm_rope_store_equals_the_separate_ops(gpu, tokens, hq, hkv, need_k):
     """qk_norm_rope_store against the sequence it replaces, both through the hip backend: bit-identical q, k
