@@ -43,11 +43,29 @@ __device__ __forceinline__ void store16_stream(void* p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
-// Sum over groups of WIDTH consecutive lanes (WIDTH a power of two <= 64); every lane gets the total.
+// The value of the lane ROT places further on inside its row of 16 lanes (wrapping): a DPP operand, no trip through the
+// LDS crossbar.
+template <int ROT>
+__device__ __forceinline__ float row_rotate(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 | ROT, 0xf, 0xf, false));   // row_ror:ROT
+}
+// Sum over groups of WIDTH consecutive lanes (WIDTH a power of two <= 64); every lane gets the total.  The steps of a
+// butterfly (partner = lane ^ off); for off < 16 the partner's value is taken from the lane `off` places around the row
+// instead, which holds the same number: the first such step pairs lanes 8 apart either way, and after each step the
+// partial sums repeat with the period of the next one, so every lane adds the same two numbers as in the butterfly.
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
+  if (WIDTH < 16) {   // groups smaller than a row: a rotation would reach into the neighbouring group
 #pragma unroll
-  for (int off = WIDTH / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    for (int off = WIDTH / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+  }
+#pragma unroll
+  for (int off = WIDTH / 2; off >= 16; off >>= 1) v += __shfl_xor(v, off, kWave);
+  v += row_rotate<8>(v);
+  v += row_rotate<4>(v);
+  v += row_rotate<2>(v);
+  v += row_rotate<1>(v);
   return v;
 }
 template <int WIDTH>

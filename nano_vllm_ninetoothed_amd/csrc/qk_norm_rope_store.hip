@@ -84,7 +84,7 @@ __global__ __launch_bounds__(kFusedThreads) void qk_norm_rope_store_kernel(
   // ---- rotary, as rotary_kernel: lanes 0..7 hold x1 pieces, lanes 8..15 the matching x2 pieces
   u32x4 other;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) other[e] = (unsigned)__shfl_xor((int)nrm[e], 8, kWave);
+  for (int e = 0; e < 4; ++e) other[e] = __float_as_uint(row_rotate<8>(__uint_as_float(nrm[e])));   // lane ^ 8 is 8 places around the row of 16
   const bool upper = lane >= 8;
   u32x4 o;
   {

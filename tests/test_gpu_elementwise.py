@@ -50,6 +50,25 @@ def test_silu_and_mul_matches_oracle(gpu, ops, rows, n):
     assert_rms_parity(got, torch.nn.functional.silu(x), y, want, "siluAndMul")
 
 
+def test_silu_and_mul_every_bf16_pattern(gpu, ops):
+    """silu depends on one bf16 input, so all 65 536 patterns can be walked: the kernel's quick route (hardware exp2 and
+    reciprocal, the exact route only near a rounding midpoint) gives the oracle's bits for every one of them, NaNs as NaNs,
+    zeros of either sign as zeros; the product with y is a single rounding on both sides."""
+    hip, ref = ops("siluAndMul")
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(64, 1024)
+    for yv in (1.0, 1.3359375, -0.75):
+        gate_up = torch.cat([x, torch.full((64, 1024), yv, dtype=torch.bfloat16)], dim=1).contiguous()
+        a, b = gate_up.chunk(2, -1)
+        want = ref(a, b)
+        ag, bg = gate_up.to(gpu).chunk(2, -1)
+        got = hip(ag, bg).cpu()
+        nan_w, nan_g = torch.isnan(want.float()), torch.isnan(got.float())
+        assert torch.equal(nan_w, nan_g)
+        same = (got.view(torch.int16) == want.view(torch.int16)) | nan_w | ((got.float() == 0) & (want.float() == 0))
+        bad = (~same).flatten().nonzero().flatten().tolist()
+        assert not bad, (yv, [hex(i) for i in bad[:8]])
+
+
 @pytest.mark.parametrize("rows,vocab", [(256, 151936), (1, 151936), (7, 1000), (33, 2048), (5, 12345)])
 def test_sampler_matches_oracle(gpu, ops, rows, vocab):
     """Greedy sampler: same token ids as argmax(softmax(logits / T)); ties resolve to the first index."""
