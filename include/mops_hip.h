@@ -302,7 +302,8 @@ int mops_hip_qk_norm_rope_store(const void* qkv, int64_t qkv_token_stride, const
  * are n and k); bias: [n] bf16 or NULL.  workspace: device scratch for solutions that split k (may be NULL
  * with workspace_bytes 0; solutions that need more than is given are not chosen).
  * The solution is the one pinned for (m, n, k) with mops_hip_linear_pin_solution if it supports the
- * problem, else the first the library's heuristic returns.  Unlike the kernels above this entry point keeps
+ * problem; without a pin for m, the one pinned for the next larger row count with the same n and k; else the
+ * first the library's heuristic returns.  Unlike the kernels above this entry point keeps
  * host-side state (a library handle per device, one descriptor per distinct shape).
  */
 int mops_hip_linear_bf16(const void* x, int64_t x_row_stride, const void* w, int64_t w_row_stride,

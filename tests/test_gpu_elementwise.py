@@ -240,3 +240,14 @@ def test_linear_with_a_pinned_solution_and_tuning(gpu):
     for y in (y0, y1, y2):
         assert (y.float() - ref).abs().max().item() <= 2 ** -7 * ref.abs().max().item() + 1e-3
     assert torch.equal(y0, y2)
+    # a row count without a pin of its own borrows the pin of the next larger one of the same weight shape (a decode step
+    # outside a graph runs any number of rows): 13 rows before, with and after a pin for 16 rows
+    x13, ref13 = x[:13], ref[:13]
+    z0 = mops.linear(x13, w)
+    assert lib.mops_hip_linear_pin_solution(m, n, k, best.value) == 0
+    z1 = mops.linear(x13, w)
+    assert lib.mops_hip_linear_pin_solution(m, n, k, -1) == 0
+    z2 = mops.linear(x13, w)
+    for z in (z0, z1, z2):
+        assert z.shape == (13, n) and (z.float() - ref13).abs().max().item() <= 2 ** -7 * ref.abs().max().item() + 1e-3
+    assert torch.equal(z0, z2)
