@@ -355,12 +355,34 @@ def load_linear_solutions(path=None) -> int:
     return len(table["solutions"])
 
 
+_linear_fn = None   # the bound C entry point, looked up once
+
+
 @register_hip_op
 def linear(x, weight, bias=None):
     """x @ weight.T (+ bias) (mops/torch/ops.py:5-7).  A library GEMM either way: bf16 problems with up to
     1024 rows (the decode step's projections, the lm head) call hipBLASLt through the C ABI, which lets a
     solution measured on cold weights be pinned per shape; everything else goes through torch."""
-    global _linear_pins_loaded
+    global _linear_pins_loaded, _linear_fn
+    # The decode step calls this 113 times with a 2-D activation and a weight seen before: what the general path below
+    # found out about the weight (shape, row stride, address, that it qualifies) is kept on the tensor, and the call is
+    # the checks that can change from call to call, the output allocation and the C call.
+    info = getattr(weight, "_mops_linear_info", None)
+    if info is not None and bias is None and x.dim() == 2:
+        n, k, ldw, wptr = info
+        m = x.shape[0]
+        if (x.dtype is torch.bfloat16 and x.is_cuda and x.shape[1] == k and 0 < m <= _LINEAR_MAX_ROWS and x.stride(1) == 1
+                and weight.data_ptr() == wptr):
+            ldx = x.stride(0) if m > 1 else k
+            xptr = x.data_ptr()
+            if ldx % 8 == 0 and xptr % 16 == 0:
+                y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+                ws = _linear_workspace(x.device)
+                st = _linear_fn(xptr, ldx, wptr, ldw, None, y.data_ptr(), n, m, n, k, ws.data_ptr(), _LINEAR_WORKSPACE_BYTES,
+                                _stream_of(x.device))
+                if st:
+                    _capi.check("mops_hip_linear_bf16", st)
+                return y
     if (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.dim() == 2
             and weight.stride(1) == 1 and x.dim() >= 1 and x.shape[-1] == weight.shape[1]
             and (bias is None or (bias.dtype == torch.bfloat16 and bias.is_contiguous() and bias.numel() == weight.shape[0]))):
@@ -376,6 +398,13 @@ def linear(x, weight, bias=None):
             if not _linear_pins_loaded:
                 _linear_pins_loaded = True
                 load_linear_solutions()
+            if _linear_fn is None:
+                _linear_fn = _capi.load().mops_hip_linear_bf16
+            if bias is None and weight.is_contiguous():
+                try:
+                    weight._mops_linear_info = (n, k, ldw, weight.data_ptr())
+                except (AttributeError, RuntimeError):
+                    pass   # a tensor that takes no attributes keeps the general path
             y = torch.empty((m, n), dtype=x.dtype, device=x.device)
             ws = _linear_workspace(x.device)
             st = _capi.load().mops_hip_linear_bf16(x2.data_ptr(), ldx, weight.data_ptr(), ldw,
